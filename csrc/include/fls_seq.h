@@ -25,7 +25,13 @@ int fls_seq_gemm(const void* A, int ta, const void* W, int tw, void* C, int tc, 
 // weights stored around zero).
 int fls_seq_group_rmsnorm(const float* x, int ldx, const int* idx, const float* w, void* y, int ty, int ldy,
                           int rows, int D, int groups, float eps, int add, float woff, fls_stream_t s);
-int fls_seq_embed(const int* ids, const void* table, int tt, float* out, int T, int D, int V, fls_stream_t s);
+// out[t] = table[ids[t]] * scale (fp32 rows of the residual stream)
+int fls_seq_embed(const int* ids, const void* table, int tt, float* out, int T, int D, int V, float scale, fls_stream_t s);
+// Dynamic Tanh norm: y[r, c] = tanh(alpha[0] x[row, c]) wb[c] + wb[D + c], row = idx ? idx[r] : r; y of type ty
+int fls_seq_dyt_norm(const float* x, int ldx, const int* idx, const float* wb, const float* alpha, void* y, int ty,
+                     int ldy, int rows, int D, fls_stream_t s);
+// x += mult * y (fp32 rows)
+int fls_seq_add_scaled(float* x, int ldx, const float* y, int ldy, int rows, int D, float mult, fls_stream_t s);
 int fls_seq_gather_rows(const void* x, int tx, int ldx, const int* idx, void* y, int ldy, int rows, int D, fls_stream_t s);
 // xIELU: z > 0: softplus(p) z^2 + z/2; else (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2; act = {p, q}
 int fls_seq_xielu(const float* z, int ldz, const float* act, void* y, int ty, int ldy, int rows, int cols, fls_stream_t s);
@@ -36,10 +42,11 @@ int fls_seq_unary(const float* z, int ldz, void* y, int ty, int ldy, int rows, i
 // per row t and head h: the n entries x[t, x_col + h x_hs ...] (x of type tx), RMS-normed over n times w[n] (w != null), the first
 // rot entries rotated in pairs (2i, 2i+1) by the angle tok_pos[t] * freqs[i]; written as type to at
 // out[row, out_col + h out_hs ...], row = row_map ? row_map[t] : t; raw (nullable, like out, row stride ldr)
-// receives the entries unchanged.  n <= 512
+// receives the entries unchanged.  unit_after != 0: after the rotation the n entries are divided by
+// sqrt(mean(entries^2) + eps), without a weight.  n <= 512
 int fls_seq_head_norm_rope(const void* x, int tx, int ldx, int x_col, int x_hs, int heads, int n, const float* w, float eps,
                            const float* freqs, int rot, const int* tok_pos, const int* row_map, void* out, int to,
-                           int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, fls_stream_t s);
+                           int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, int unit_after, fls_stream_t s);
 int fls_seq_softcap(float* z, int ldz, int rows, int cols, float cap, fls_stream_t s);
 int fls_seq_argmax(const float* z, int ldz, int rows, int cols, int* out, fls_stream_t s);
 // k rows RMS-normed over all kcols (times kn), k and v rows written at row kv_slot[r] of the pools
@@ -53,13 +60,15 @@ int fls_seq_kv_store(const float* k, int ldk, const float* kn, float eps, const 
 // columns of pool rows ldk / ldv wide (both may be one pool).  q of type tq (fp32 allowed over bf16 pools),
 // pools and out of type tc.  out = result * out_scale.  nsplit > 1: every row's keys are cut into nsplit
 // ranges that run as blocks of their own (few rows, many keys: decoding) and are merged by a second
-// kernel; part: T H nsplit (dv + 4) floats of scratch (16-byte aligned).
+// kernel; part: T H nsplit (dv + 4) floats of scratch (16-byte aligned).  has_sink != 0 (softmax only): one more
+// entry of score `sink` and no value joins the softmax's sum.  head_gate (nullable) [T, H] fp32, row stride ldhg:
+// the output of (row, head) times sigmoid(head_gate[t, h]).
 int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, int tc,
                        void* out, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
                        int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
                        const float* r1, const float* r2, int chunk, int window, int keep_first,
                        const float* gate_bias, float out_scale, int page_size, int nsplit, float* part,
-                       fls_stream_t s);
+                       int has_sink, float sink, const float* head_gate, int ldhg, fls_stream_t s);
 // the same attention on the matrix cores for bf16 pools and rows in tiles: tiles[n_tiles][2] = (first packed
 // row, rows <= 128) of one request each, covering every row of the step; q of type tq.  -2: shape not
 // served (use the above)
@@ -67,7 +76,8 @@ int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* kc, int ldk
                          int ldo, const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
                          const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
                          float softcap, const float* r1, const float* r2, int chunk, int window, int keep_first,
-                         const float* gate_bias, float out_scale, int page_size, fls_stream_t s);
+                         const float* gate_bias, float out_scale, int page_size, int has_sink, float sink,
+                         const float* head_gate, int ldhg, fls_stream_t s);
 // softmax attention of few rows whose H / G <= 32 query heads per key / value head become the columns of one
 // matrix-core tile (decode steps over cached latent rows): fp32 q, bf16 pools and out, window and kept first
 // keys as above; nsplit ranges of key tiles per row, part: T H nsplit (dv + 4) floats.  -2: shape not served
@@ -111,7 +121,8 @@ int fls_seq_ssd_scan(const float* xbc, int ldx, const float* z, int ldz, const f
                      const int* cu, const int* pos0, const int* slot, int B, int nh, int P, int N, int G,
                      fls_stream_t s);
 // softmax scores over E experts; the top largest of (score + corr) chosen (ties: the lower expert);
-// ids[T, top], w[T, top] = bare scores; hist[E] += number of entries per expert (hist zeroed by the caller)
+// ids[T, top], w[T, top] = bare scores; hist[E] += number of entries per expert (hist zeroed by the caller).
+// corr == null: the top largest logits are chosen and w = the softmax over the chosen logits only
 int fls_seq_moe_route(const float* logits, int ldl, const float* corr, int T, int E, int top, int* ids, float* w,
                       int* hist, fls_stream_t s);
 // offs[E+1] = exclusive scan of hist; cursor[E] = offs[:E]
@@ -121,6 +132,9 @@ int fls_seq_moe_place(const int* ids, int n, int top, int* cursor, int* dest, in
 // out[t] = sum_k w[t, k] y[dest[t, k]] (fp32, k in order)
 int fls_seq_moe_sum(const float* y, int ldy, const int* dest, const float* w, float* out, int ldo, int T, int top,
                     int D, fls_stream_t s);
+// x[t] += mult * (sum_k w[t, k] y[dest[t, k]] + sigmoid(gate[t * ldg]) shared[t]); shared nullable, gate nullable (then 1)
+int fls_seq_moe_combine(float* x, int ldx, const float* y, int ldy, const int* dest, const float* w, int T, int top,
+                        const float* shared, int lds, const float* gate, int ldg, int D, float mult, fls_stream_t s);
 #ifdef __cplusplus
 }
 #endif

@@ -3,7 +3,9 @@
 // own.  Visible: j <= i inside the row's chunk and / or window, plus, with keep_first, the first
 // keep_first keys of the sequence however far back they lie.  Keys and values are the first G d and
 // G dv columns of pool rows ldk and ldv wide, so both may be one pool (values = a prefix of the keys:
-// attention over latent rows).  The query may be fp32 while the pools hold bf16.
+// attention over latent rows).  The query may be fp32 while the pools hold bf16.  has_sink: the softmax
+// has one more entry of score `sink` and no value (p_j = exp(s_j) / (exp(sink) + sum exp(s))); head_gate
+// [T, H] fp32: the output of (row, head) times sigmoid(head_gate[t, h]).
 //
 // One block (four wavefronts) per (row, query head).  The row's query sits in LDS as fp32.  The keys
 // it may see -- j <= i, inside its chunk of the sequence and / or its window -- are walked in tiles of
@@ -56,7 +58,8 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
                                                          const float* __restrict__ r1, const float* __restrict__ r2,
                                                          int chunk, int window, int keep_first,
                                                          const float* __restrict__ gate_bias, float out_scale,
-                                                         int page_size, int vec, float* __restrict__ part) {
+                                                         int page_size, int vec, float* __restrict__ part, int has_sink,
+                                                         float sink, const float* __restrict__ head_gate, int ldhg) {
   __shared__ float qs[MAX_D];
   __shared__ float pw[4][64];
   __shared__ int prow[4][64];
@@ -145,10 +148,13 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
       for (int w = 0; w < 4; ++w) f[w] = 1.f;
     } else {
       mx = fmaxf(fmaxf(mm[0], mm[1]), fmaxf(mm[2], mm[3]));
+      if (has_sink && nsplit == 1) mx = fmaxf(mx, sink);          // (with ranges the merge adds the silent entry, once)
 #pragma unroll
       for (int w = 0; w < 4; ++w) { f[w] = expf(mm[w] - mx); lt += ll[w] * f[w]; }
+      if (has_sink && nsplit == 1) lt += expf(sink - mx);
       inv = out_scale / lt;
     }
+    if (head_gate != nullptr) inv *= sigmoid_f(head_gate[(size_t)t * ldhg + h]);
     if (nsplit > 1) {                              // this range's share, not yet normalised
       float* pp = part + (((size_t)t * H + h) * nsplit + blockIdx.z) * (dv + 4);      // record: values[dv] | maximum | sum | pad
       if (lane == 0) { pp[dv] = mx; pp[dv + 1] = lt; }
@@ -176,7 +182,7 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
 #define MERGE_MAX_SPLIT 64
 template <typename T>
 __global__ void attn_merge_kernel(const float* __restrict__ part, T* __restrict__ out, int ldo, int H, int dv, int nsplit, int gated,
-                                  float out_scale) {
+                                  float out_scale, int has_sink, float sink, const float* __restrict__ head_gate, int ldhg) {
   __shared__ float wz[MERGE_MAX_SPLIT];
   const int t = blockIdx.y, h = blockIdx.x;
   const int rs = dv + 4;                           // record: values[dv] | maximum | sum | pad
@@ -185,10 +191,13 @@ __global__ void attn_merge_kernel(const float* __restrict__ part, T* __restrict_
     const int z = threadIdx.x;
     const float mz = (z < nsplit && !gated) ? pp[z * rs + dv] : -1e30f;
     const float lz = (z < nsplit && !gated) ? pp[z * rs + dv + 1] : 0.f;
-    const float mx = wave_max(mz);
+    float mx = wave_max(mz);
+    if (has_sink) mx = fmaxf(mx, sink);
     const float f = expf(mz - mx);
-    const float lt = wave_sum(lz * f);
-    wz[z] = gated ? out_scale : f * out_scale / lt;
+    float lt = wave_sum(lz * f);
+    if (has_sink) lt += expf(sink - mx);
+    const float os = head_gate != nullptr ? out_scale * sigmoid_f(head_gate[(size_t)t * ldhg + h]) : out_scale;
+    wz[z] = gated ? os : f * os / lt;
   }
   __syncthreads();
   for (int e = threadIdx.x; e < dv; e += blockDim.x) {
@@ -200,11 +209,11 @@ __global__ void attn_merge_kernel(const float* __restrict__ part, T* __restrict_
 
 // (also used by the matrix-core kernels that cut a row's keys over blocks)
 int seq_attn_merge(const float* part, void* out, int tc, int ldo, int T, int H, int dv, int nsplit, int gated, float out_scale,
-                   fls_stream_t s) {
+                   int has_sink, float sink, const float* head_gate, int ldhg, fls_stream_t s) {
   const int threads = dv > 128 ? 256 : (dv > 64 ? 128 : 64);
   hipStream_t st = (hipStream_t)s;
-  if (tc == 1) hipLaunchKernelGGL((attn_merge_kernel<bf16_t>), dim3(H, T), dim3(threads), 0, st, part, (bf16_t*)out, ldo, H, dv, nsplit, gated, out_scale);
-  else hipLaunchKernelGGL((attn_merge_kernel<float>), dim3(H, T), dim3(threads), 0, st, part, (float*)out, ldo, H, dv, nsplit, gated, out_scale);
+  if (tc == 1) hipLaunchKernelGGL((attn_merge_kernel<bf16_t>), dim3(H, T), dim3(threads), 0, st, part, (bf16_t*)out, ldo, H, dv, nsplit, gated, out_scale, has_sink, sink, head_gate, ldhg);
+  else hipLaunchKernelGGL((attn_merge_kernel<float>), dim3(H, T), dim3(threads), 0, st, part, (float*)out, ldo, H, dv, nsplit, gated, out_scale, has_sink, sink, head_gate, ldhg);
   SEQ_LAUNCH_CHECK();
   return 0;
 }
@@ -215,15 +224,17 @@ extern "C" int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc
                                   int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
                                   const float* r1, const float* r2, int chunk, int window, int keep_first,
                                   const float* gate_bias, float out_scale, int page_size, int nsplit, float* part,
-                                  fls_stream_t s) {
+                                  int has_sink, float sink, const float* head_gate, int ldhg, fls_stream_t s) {
   if (T <= 0) return 0;
+  if (has_sink && gate_bias != nullptr) return -1;      // (a silent entry belongs to a softmax)
   if (nsplit < 1 || nsplit > MERGE_MAX_SPLIT || (nsplit > 1 && part == nullptr)) return -1;
   if (d > MAX_D || dv > 64 * MAX_DV_PER_LANE || G < 1 || H % G || page_size < 1 || G * d > ldk || G * dv > ldv || keep_first < 0
       || (tq == 1 && tc == 0)) return -1;
   dim3 grid(H, T, nsplit);
   hipStream_t st = (hipStream_t)s;
 #define ATTN_PAGED_ARGS ldq, (const TC*)kc, ldk, (const TC*)vc, ldv, (TC*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, \
-                        d, dv, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias, out_scale, page_size, vec, part
+                        d, dv, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias, out_scale, page_size, vec, part, has_sink, sink, \
+                        nsplit > 1 ? nullptr : head_gate, ldhg
   if (tc == 1) {
     using TC = bf16_t;
     const int vec = d % 8 == 0 && (uintptr_t)kc % 16 == 0 && ldk % 8 == 0;
@@ -236,6 +247,6 @@ extern "C" int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc
   }
 #undef ATTN_PAGED_ARGS
   SEQ_LAUNCH_CHECK();
-  if (nsplit > 1) return seq_attn_merge(part, out, tc, ldo, T, H, dv, nsplit, gate_bias != nullptr, out_scale, s);
+  if (nsplit > 1) return seq_attn_merge(part, out, tc, ldo, T, H, dv, nsplit, gate_bias != nullptr, out_scale, has_sink, sink, head_gate, ldhg, s);
   return 0;
 }

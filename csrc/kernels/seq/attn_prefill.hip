@@ -35,7 +35,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const TQ* __restrict_
                                                            int pt_stride, int H, int G, float scale, float softcap,
                                                            const float* __restrict__ r1, const float* __restrict__ r2,
                                                            int chunk, int window, int keep_first,
-                                                           const float* __restrict__ gate_bias, float out_scale, int page_size) {
+                                                           const float* __restrict__ gate_bias, float out_scale, int page_size,
+                                                           int has_sink, float sink, const float* __restrict__ head_gate,
+                                                           int ldhg) {
   constexpr int KLD = D + 8;
   __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t Vt[DV * PLD];
@@ -82,7 +84,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const TQ* __restrict_
   for (int c = 0; c < DV / 32; ++c)
 #pragma unroll
     for (int r = 0; r < 16; ++r) O[c][r] = 0.f;
-  float m = -1e30f, l = 0.f;
+  // (the softmax's silent entry of score `sink`, if any, is where every query's running maximum and sum start)
+  float m = has_sink ? sink : -1e30f, l = has_sink ? 1.f : 0.f;
   const float a1 = r1 != nullptr ? r1[h] : 0.f, a2 = r2 != nullptr ? r2[h] : 0.f;
   const bool gated = gate_bias != nullptr;
   const float gb = gated ? gate_bias[h] : 0.f;
@@ -213,7 +216,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const TQ* __restrict_
     __builtin_amdgcn_wave_barrier();
   }
   if (qok && (gated || l > 0.f)) {
-    const float inv = gated ? out_scale : out_scale / l;
+    float inv = gated ? out_scale : out_scale / l;
+    if (head_gate != nullptr) inv *= sigmoid_f(head_gate[(size_t)(row0 + qrow) * ldhg + h]);
     bf16_t* op = out + (size_t)(row0 + qrow) * ldo + (size_t)h * DV;
 #pragma unroll
     for (int c = 0; c < DV / 32; ++c)
@@ -234,8 +238,10 @@ extern "C" int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* 
                                     int ldo, const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
                                     const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
                                     float softcap, const float* r1, const float* r2, int chunk, int window, int keep_first,
-                                    const float* gate_bias, float out_scale, int page_size, fls_stream_t s) {
+                                    const float* gate_bias, float out_scale, int page_size, int has_sink, float sink,
+                                    const float* head_gate, int ldhg, fls_stream_t s) {
   if (n_tiles <= 0) return 0;
+  if (has_sink && gate_bias != nullptr) return -1;
   if (G < 1 || H % G || page_size < 1 || ldq % 8 || ldo % 4 || ldk % 8 || ldv % 8 || G * d > ldk || G * dv > ldv ||
       (uintptr_t)q % 16 || (uintptr_t)kc % 16 || (uintptr_t)vc % 16 || (uintptr_t)out % 8 || keep_first < 0)
     return -2;
@@ -247,12 +253,12 @@ extern "C" int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* 
       hipLaunchKernelGGL((attn_prefill_kernel<DD, DDV, bf16_t>), grid, dim3(256), 0, st, (const bf16_t*)q, ldq,           \
                          (const bf16_t*)kc, ldk, (const bf16_t*)vc, ldv, (bf16_t*)out, ldo, tiles, tok_seq, tok_pos,      \
                          page_table, pt_stride, H, G, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias,       \
-                         out_scale, page_size);                                                                           \
+                         out_scale, page_size, has_sink, sink, head_gate, ldhg);                                          \
     else                                                                                                                  \
       hipLaunchKernelGGL((attn_prefill_kernel<DD, DDV, float>), grid, dim3(256), 0, st, (const float*)q, ldq,             \
                          (const bf16_t*)kc, ldk, (const bf16_t*)vc, ldv, (bf16_t*)out, ldo, tiles, tok_seq, tok_pos,      \
                          page_table, pt_stride, H, G, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias,       \
-                         out_scale, page_size);                                                                           \
+                         out_scale, page_size, has_sink, sink, head_gate, ldhg);                                          \
   } while (0)
   if (d == 128 && dv == 128) ATTN_PF(128, 128);
   else if (d == 64 && dv == 64) ATTN_PF(64, 64);
@@ -476,6 +482,6 @@ extern "C" int fls_seq_attn_heads(const void* q, int ldq, const void* kc, int ld
   else return -2;
 #undef ATTN_HEADS
   SEQ_LAUNCH_CHECK();
-  if (nsplit > 1) return seq_attn_merge(part, out, 1, ldo, T, H, dv, nsplit, 0, out_scale, s);
+  if (nsplit > 1) return seq_attn_merge(part, out, 1, ldo, T, H, dv, nsplit, 0, out_scale, 0, 0.f, nullptr, 0, s);
   return 0;
 }

@@ -39,20 +39,90 @@ extern "C" int fls_seq_group_rmsnorm(const float* x, int ldx, const int* idx, co
   return 0;
 }
 
+// ------------------------------------------------------------------------- Dynamic Tanh norm
+// y[r, c] = tanh(alpha x[row, c]) w[c] + b[c]: no statistic of the row, so the work is cut over
+// (row, 1024-column piece) blocks of four columns a thread.  wb = [w; b], alpha one number on the device.
+template <typename TO>
+__global__ __launch_bounds__(256) void dyt_norm_kernel(const float* __restrict__ x, int ldx, const int* __restrict__ idx,
+                                                       const float* __restrict__ wb, const float* __restrict__ alpha,
+                                                       TO* __restrict__ y, int ldy, int D, int vec) {
+  const int r = blockIdx.x;
+  const float a = alpha[0];
+  const float* xr = x + (size_t)(idx != nullptr ? idx[r] : r) * ldx;
+  const float* w = wb;
+  const float* b = wb + D;
+  TO* yr = y + (size_t)r * ldy;
+  const int c0 = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c0 >= D) return;
+  if (vec) {
+    const float4 v = *reinterpret_cast<const float4*>(xr + c0);
+    const float4 wv = *reinterpret_cast<const float4*>(w + c0), bv = *reinterpret_cast<const float4*>(b + c0);
+    const float o0 = tanhf(a * v.x) * wv.x + bv.x, o1 = tanhf(a * v.y) * wv.y + bv.y;
+    const float o2 = tanhf(a * v.z) * wv.z + bv.z, o3 = tanhf(a * v.w) * wv.w + bv.w;
+    if constexpr (sizeof(TO) == 2) {
+      bf16_t e[4] = {f_to_bf16(o0), f_to_bf16(o1), f_to_bf16(o2), f_to_bf16(o3)};
+      *reinterpret_cast<uint2*>(yr + c0) = *reinterpret_cast<const uint2*>(e);
+    } else {
+      *reinterpret_cast<float4*>(yr + c0) = make_float4(o0, o1, o2, o3);
+    }
+  } else {
+    for (int c = c0; c < min(D, c0 + 4); ++c) stf(yr, c, tanhf(a * xr[c]) * w[c] + b[c]);
+  }
+}
+
+extern "C" int fls_seq_dyt_norm(const float* x, int ldx, const int* idx, const float* wb, const float* alpha, void* y, int ty,
+                                int ldy, int rows, int D, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  if (D < 1) return -1;
+  const int vec = D % 4 == 0 && ldx % 4 == 0 && ldy % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)wb % 16 == 0 &&
+                  (uintptr_t)y % 16 == 0;
+  dim3 grid(rows, (D + 1023) / 1024);
+  hipStream_t st = (hipStream_t)s;
+  if (ty == 1) hipLaunchKernelGGL((dyt_norm_kernel<bf16_t>), grid, dim3(256), 0, st, x, ldx, idx, wb, alpha, (bf16_t*)y, ldy, D, vec);
+  else hipLaunchKernelGGL((dyt_norm_kernel<float>), grid, dim3(256), 0, st, x, ldx, idx, wb, alpha, (float*)y, ldy, D, vec);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// x[r, c] += mult * y[r, c]: a sublayer's output joins the residual stream scaled
+__global__ __launch_bounds__(256) void add_scaled_kernel(float* __restrict__ x, int ldx, const float* __restrict__ y, int ldy, int D,
+                                                         float mult, int vec) {
+  float* xr = x + (size_t)blockIdx.x * ldx;
+  const float* yr = y + (size_t)blockIdx.x * ldy;
+  const int c0 = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c0 >= D) return;
+  if (vec) {
+    float4 a = *reinterpret_cast<const float4*>(xr + c0);
+    const float4 b = *reinterpret_cast<const float4*>(yr + c0);
+    a.x += mult * b.x; a.y += mult * b.y; a.z += mult * b.z; a.w += mult * b.w;
+    *reinterpret_cast<float4*>(xr + c0) = a;
+  } else {
+    for (int c = c0; c < min(D, c0 + 4); ++c) xr[c] += mult * yr[c];
+  }
+}
+
+extern "C" int fls_seq_add_scaled(float* x, int ldx, const float* y, int ldy, int rows, int D, float mult, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  const int vec = D % 4 == 0 && ldx % 4 == 0 && ldy % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0;
+  hipLaunchKernelGGL(add_scaled_kernel, dim3(rows, (D + 1023) / 1024), dim3(256), 0, (hipStream_t)s, x, ldx, y, ldy, D, mult, vec);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ------------------------------------------------------------------------------- embedding
 template <typename T>
-__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int D, int V) {
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int D, int V, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= V ? V - 1 : id);
   const T* row = table + (size_t)id * D;
-  for (int c = threadIdx.x; c < D; c += blockDim.x) out[(size_t)t * D + c] = ldf(row, c);
+  for (int c = threadIdx.x; c < D; c += blockDim.x) out[(size_t)t * D + c] = ldf(row, c) * scale;
 }
 
-extern "C" int fls_seq_embed(const int* ids, const void* table, int tt, float* out, int T, int D, int V, fls_stream_t s) {
+extern "C" int fls_seq_embed(const int* ids, const void* table, int tt, float* out, int T, int D, int V, float scale, fls_stream_t s) {
   if (T <= 0) return 0;
-  if (tt == 1) hipLaunchKernelGGL((embed_kernel<bf16_t>), dim3(T), dim3(256), 0, (hipStream_t)s, ids, (const bf16_t*)table, out, D, V);
-  else hipLaunchKernelGGL((embed_kernel<float>), dim3(T), dim3(256), 0, (hipStream_t)s, ids, (const float*)table, out, D, V);
+  if (tt == 1) hipLaunchKernelGGL((embed_kernel<bf16_t>), dim3(T), dim3(256), 0, (hipStream_t)s, ids, (const bf16_t*)table, out, D, V, scale);
+  else hipLaunchKernelGGL((embed_kernel<float>), dim3(T), dim3(256), 0, (hipStream_t)s, ids, (const float*)table, out, D, V, scale);
   SEQ_LAUNCH_CHECK();
   return 0;
 }
@@ -215,7 +285,7 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(const TI* x, int ld
                                                              const float* __restrict__ freqs, int rot,
                                                              const int* __restrict__ tok_pos, const int* __restrict__ row_map,
                                                              TO* out, int ldo, int out_col, int out_hs, TO* raw, int ldr,
-                                                             int items) {
+                                                             int items, int unit_after) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (item >= items) return;
@@ -252,20 +322,30 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(const TI* x, int ld
       const float cs = cosf(ang), sn = sinf(ang);
       val = (c & 1) ? v[e] * cs + other * sn : v[e] * cs - other * sn;
     }
-    if (c < n) stf(orow, c, val);
+    if (!unit_after) { if (c < n) stf(orow, c, val); }
+    else v[e] = val;
+  }
+  if (unit_after) {                                  // (block-uniform)
+    float s2 = 0.f;
+#pragma unroll
+    for (int e = 0; e < HNR_MAX_E; ++e) s2 += v[e] * v[e];          // (entries past n are zeros)
+    const float rs = 1.f / sqrtf(wave_sum(s2) / (float)n + eps);
+#pragma unroll
+    for (int e = 0; e < HNR_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) stf(orow, c, v[e] * rs); }
   }
 }
 
 extern "C" int fls_seq_head_norm_rope(const void* x, int tx, int ldx, int x_col, int x_hs, int heads, int n, const float* w,
                                       float eps, const float* freqs, int rot, const int* tok_pos, const int* row_map, void* out,
-                                      int to, int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, fls_stream_t s) {
+                                      int to, int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, int unit_after,
+                                      fls_stream_t s) {
   if (rows <= 0 || heads <= 0) return 0;
   if (n < 1 || n > 64 * HNR_MAX_E || rot < 0 || rot > n || (rot & 1) || (rot > 0 && (freqs == nullptr || tok_pos == nullptr))) return -1;
   const int items = rows * heads;
   dim3 grid((items + 3) / 4);
   hipStream_t st = (hipStream_t)s;
 #define HNR(TI, TO) hipLaunchKernelGGL((head_norm_rope_kernel<TI, TO>), grid, dim3(256), 0, st, (const TI*)x, ldx, x_col, x_hs, heads, \
-                                       n, w, eps, freqs, rot, tok_pos, row_map, (TO*)out, ldo, out_col, out_hs, (TO*)raw, ldr, items)
+                                       n, w, eps, freqs, rot, tok_pos, row_map, (TO*)out, ldo, out_col, out_hs, (TO*)raw, ldr, items, unit_after)
   if (tx == 1 && to == 1) HNR(bf16_t, bf16_t);
   else if (tx == 1) HNR(bf16_t, float);
   else if (to == 1) HNR(float, bf16_t);
@@ -276,13 +356,40 @@ extern "C" int fls_seq_head_norm_rope(const void* x, int tx, int ldx, int x_col,
 }
 
 // ------------------------------------------------------------------------ mixture of experts
-// one thread per token: softmax statistics, then `top` passes each taking the best unchosen expert
+// one thread per token: softmax statistics, then `top` passes each taking the best unchosen expert.
+// corr == null: the `top` largest logits are chosen (ties: the lower expert) and weighted by the softmax
+// over the chosen logits only
 #define MOE_MAX_TOP 16
 __global__ void moe_route_kernel(const float* __restrict__ logits, int ldl, const float* __restrict__ corr, int T, int E, int top,
                                  int* __restrict__ ids, float* __restrict__ w, int* __restrict__ hist) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const float* l = logits + (size_t)t * ldl;
+  if (corr == nullptr) {
+    int chosen[MOE_MAX_TOP];
+    float val[MOE_MAX_TOP];
+    for (int k = 0; k < top; ++k) {
+      float best = -INFINITY;
+      int be = -1;
+      for (int e = 0; e < E; ++e) {
+        bool used = false;
+        for (int j = 0; j < k; ++j) used |= (chosen[j] == e);
+        if (used) continue;
+        const float c = l[e];
+        if (be < 0 || c > best) { best = c; be = e; }
+      }
+      chosen[k] = be;
+      val[k] = best;
+    }
+    float sum = 0.f;                                  // val[0] is the largest
+    for (int k = 0; k < top; ++k) { val[k] = expf(val[k] - val[0]); sum += val[k]; }
+    const float inv = 1.f / sum;
+    for (int k = 0; k < top; ++k) {
+      ids[(size_t)t * top + k] = chosen[k];
+      w[(size_t)t * top + k] = val[k] * inv;
+    }
+    return;
+  }
   float mx = -INFINITY;
   for (int e = 0; e < E; ++e) mx = fmaxf(mx, l[e]);
   float sum = 0.f;
@@ -393,4 +500,28 @@ extern "C" int fls_seq_moe_sum(const float* y, int ldy, const int* dest, const f
   return 0;
 }
 
-extern "C" int fls_seq_version(void) { return 7; }
+// x[t, c] += mult * (sum_k w[t, k] y[dest[t, k], c] + sigmoid(gate[t]) shared[t, c]); shared / gate nullable
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, int ldx, const float* __restrict__ y, int ldy,
+                                                          const int* __restrict__ dest, const float* __restrict__ w, int top,
+                                                          const float* __restrict__ shared, int lds, const float* __restrict__ gate,
+                                                          int ldg, int D, float mult) {
+  const int t = blockIdx.x;
+  const float sg = shared == nullptr ? 0.f : (gate != nullptr ? sigmoid_f(gate[(size_t)t * ldg]) : 1.f);
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < D; c += 256 * gridDim.y) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) acc += w[(size_t)t * top + k] * y[(size_t)dest[(size_t)t * top + k] * ldy + c];
+    if (shared != nullptr) acc += sg * shared[(size_t)t * lds + c];
+    x[(size_t)t * ldx + c] += mult * acc;
+  }
+}
+
+extern "C" int fls_seq_moe_combine(float* x, int ldx, const float* y, int ldy, const int* dest, const float* w, int T, int top,
+                                   const float* shared, int lds, const float* gate, int ldg, int D, float mult, fls_stream_t s) {
+  if (T <= 0) return 0;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, (D + 1023) / 1024), dim3(256), 0, (hipStream_t)s, x, ldx, y, ldy, dest, w, top, shared,
+                     lds, gate, ldg, D, mult);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int fls_seq_version(void) { return 8; }

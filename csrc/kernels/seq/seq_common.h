@@ -45,7 +45,8 @@ __device__ __forceinline__ float gelu_tanh_f(float z) {
 
 // attn_paged.hip: out[t, h] from nsplit partial (maximum, sum, weighted values) records per (row, head)
 typedef void* fls_stream_t;
+// has_sink: the softmax's silent entry of score `sink` joins the total here; head_gate (nullable) [T, H]: a sigmoid gate per (row, head)
 int seq_attn_merge(const float* part, void* out, int tc, int ldo, int T, int H, int dv, int nsplit, int gated, float out_scale,
-                   fls_stream_t s);
+                   int has_sink, float sink, const float* head_gate, int ldhg, fls_stream_t s);
 
 #define SEQ_LAUNCH_CHECK() do { hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return (int)e_; } while (0)

@@ -130,7 +130,7 @@ def _load_kernels(path: str = _KERNELS):
     return lib
 
 
-SEQ_ABI = 7   # csrc/include/fls_seq.h
+SEQ_ABI = 8   # csrc/include/fls_seq.h
 
 
 def _load_seq():
@@ -142,18 +142,23 @@ def _load_seq():
     p, i, f, ll = c_void_p, c_int, c_float, ctypes.c_longlong
     _bind(lib, "fls_seq_gemm", i, p, i, p, i, p, i, p, p, i, i, i, i, i, i, i, p, ll, i, ll, ll, p)
     _bind(lib, "fls_seq_group_rmsnorm", i, p, i, p, p, p, i, i, i, i, i, f, i, f, p)
-    _bind(lib, "fls_seq_embed", i, p, p, i, p, i, i, i, p)
+    _bind(lib, "fls_seq_embed", i, p, p, i, p, i, i, i, f, p)
+    _bind(lib, "fls_seq_dyt_norm", i, p, i, p, p, p, p, i, i, i, i, p)
+    _bind(lib, "fls_seq_add_scaled", i, p, i, p, i, i, i, f, p)
+    _bind(lib, "fls_seq_moe_combine", i, p, i, p, i, p, p, i, i, p, i, p, i, i, f, p)
     _bind(lib, "fls_seq_gather_rows", i, p, i, i, p, p, i, i, i, p)
     _bind(lib, "fls_seq_xielu", i, p, i, p, p, i, i, i, i, p)
     _bind(lib, "fls_seq_gate_mul", i, p, i, p, i, i, i, i, i, p)
     _bind(lib, "fls_seq_unary", i, p, i, p, i, i, i, i, i, p)
-    _bind(lib, "fls_seq_head_norm_rope", i, p, i, i, i, i, i, i, p, f, p, i, p, p, p, i, i, i, i, p, i, i, p)
+    _bind(lib, "fls_seq_head_norm_rope", i, p, i, i, i, i, i, i, p, f, p, i, p, p, p, i, i, i, i, p, i, i, i, p)
     _bind(lib, "fls_seq_delta_rule_scan", i, p, i, p, i, p, i, p, i, p, i, p, i, p, p, p, p, i, i, p, p, p, i, i, i, i, f, f, f, f, i, p, p)
     _bind(lib, "fls_seq_softcap", i, p, i, i, i, f, p)
     _bind(lib, "fls_seq_argmax", i, p, i, i, i, p, p)
     _bind(lib, "fls_seq_kv_store", i, p, i, p, f, p, i, p, p, i, p, i, i, i, p)
-    _bind(lib, "fls_seq_attn_paged", i, p, i, i, p, i, p, i, i, p, i, p, p, p, i, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i, i, p, p)
-    _bind(lib, "fls_seq_attn_prefill", i, p, i, i, p, i, p, i, p, i, p, i, p, p, p, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i, p)
+    _bind(lib, "fls_seq_attn_paged", i, p, i, i, p, i, p, i, i, p, i, p, p, p, i, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i, i, p,
+          i, f, p, i, p)
+    _bind(lib, "fls_seq_attn_prefill", i, p, i, i, p, i, p, i, p, i, p, i, p, p, p, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i,
+          i, f, p, i, p)
     _bind(lib, "fls_seq_attn_heads", i, p, i, p, i, p, i, p, i, p, p, p, i, i, i, i, i, i, f, i, i, f, i, i, p, p)
     _bind(lib, "fls_seq_causal_conv", i, p, i, p, p, p, p, i, i, p, p, p, p, i, i, i, i, i, i, i, p)
     _bind(lib, "fls_seq_rglru_scan", i, p, i, p, i, p, p, i, p, p, i, i, p, p, p, i, i, f, p)

@@ -647,8 +647,92 @@ class SisavikConfig:
                 "layers": [{"type": l.type, "mixer": l.mixer, "mlp": l.mlp} for l in self.layers]}
 
 
+@dataclass
+class GizezenConfig:
+    """Gizezen: a pre-norm decoder of sliding-window attention layers with mixture-of-experts
+    feed-forwards.  x <- x + m * mixer(N1(x)), x <- x + m * ff(N2(x)) with m = ``residual_mult`` and N
+    a Dynamic Tanh norm, tanh(alpha x) w + b (no row statistics).  The attention runs a short causal
+    convolution over q, k and v right after their projections, rotates pairs of q and k (frequencies
+    optionally rescaled by wavelength, ``rot.scaling``), divides them by their root mean square per
+    head, adds a silent key of score 0 to the softmax, and gates each head's output by a sigmoid of the
+    layer's input; a layer with ``kv_from`` reads another layer's cached keys and values.  The
+    feed-forward picks ``router.top`` experts by their logits (softmax over the chosen) and may add a
+    sigmoid-gated shared expert.  Everything is read from config.json: ``width``, ``vocab``,
+    ``norm.eps``, ``residual_mult``, ``embedding.scale`` and ``layers`` (per layer ``type``, ``mixer``
+    sizes, ``mlp``)."""
+    width: int
+    vocab: int
+    norm_eps: float
+    residual_mult: float
+    embedding_scale: float
+    layers: list
+    family = "gizezen"
+    model_type = "gizezen"
+    is_moe = False
+    sliding_window = None
+    tie_word_embeddings = False
+
+    hidden_size = KagolixConfig.hidden_size
+    vocab_size = KagolixConfig.vocab_size
+    num_hidden_layers = KagolixConfig.num_hidden_layers
+    num_layers_total = KagolixConfig.num_layers_total
+    layer_names = KagolixConfig.layer_names
+    layer = KagolixConfig.layer
+    save = KagolixConfig.save
+    total_params = KagolixConfig.total_params
+
+    def kv_owner(self, i: int) -> int:
+        """The layer whose cached keys and values layer ``i`` reads (itself unless it names ``kv_from``)."""
+        j = self.layers[i].mixer.get("kv_from")
+        return i if j is None else int(j)
+
+    def validate(self) -> None:
+        for i, l in enumerate(self.layers):
+            m = l.mixer
+            if l.type != "attention":
+                raise NotImplementedError(f"layer {i}: mixer type {l.type!r}")
+            if m["heads"] % m["kv_heads"]:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+            if int(m.get("conv", 1)) < 1:
+                raise ValueError(f"layer {i}: conv must be >= 1 taps")
+            rot = m.get("rot")
+            if rot is not None and (int(rot["dims"]) > m["dim"] or int(rot["dims"]) % 2):
+                raise ValueError(f"layer {i}: rot.dims must be even and at most dim")
+            if m.get("mask") is not None and int(m["mask"]["size"]) < 1:
+                raise ValueError(f"layer {i}: mask.size must be >= 1")
+            if m["dim"] > 512 or m["vdim"] > 512:
+                # (head_norm_rope keeps a head in one wave's registers, the paged attention 8 value columns a lane)
+                raise NotImplementedError(f"layer {i}: head sizes above 512")
+            j = m.get("kv_from")
+            if j is not None:
+                o = self.layers[int(j)] if 0 <= int(j) < i else None
+                if o is None or o.mixer.get("kv_from") is not None:
+                    raise ValueError(f"layer {i}: kv_from must name an earlier layer with keys and values of its own")
+                if any(o.mixer[k] != m[k] for k in ("kv_heads", "dim", "vdim")) or o.mixer.get("rot") != m.get("rot"):
+                    raise ValueError(f"layer {i}: kv_heads, dim, vdim and rotation must equal layer {j}'s")
+            if l.mlp is not None:
+                if l.mlp.get("kind", "moe") != "moe":
+                    raise NotImplementedError(f"layer {i}: mlp kind {l.mlp['kind']!r}")
+                r = l.mlp["router"]
+                if not 1 <= r["top"] <= min(r["experts"], 16) or r["experts"] > 1024:
+                    raise NotImplementedError(f"layer {i}: router {r}")
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "GizezenConfig":
+        layers = [HybridLayer(l["type"], json.loads(json.dumps(l["mixer"])),
+                              None if l.get("mlp") is None else json.loads(json.dumps(l["mlp"]))) for l in d["layers"]]
+        cfg = cls(int(d["width"]), int(d["vocab"]), float(d["norm"]["eps"]), float(d.get("residual_mult", 1.0)),
+                  float((d.get("embedding") or {}).get("scale", 1.0)), layers)
+        cfg.validate()
+        return cfg
+
+    def to_dict(self) -> dict:
+        return {"architecture": "Gizezen", "width": self.width, "vocab": self.vocab, "norm": {"eps": self.norm_eps},
+                "residual_mult": self.residual_mult, "embedding": {"scale": self.embedding_scale},
+                "layers": [{"type": l.type, "mixer": l.mixer, "mlp": l.mlp} for l in self.layers]}
+
 # "architecture" of config.json -> config class of a stateful hybrid family
-ARCHITECTURES = {"Kagolix": KagolixConfig, "Sisavik": SisavikConfig}
+ARCHITECTURES = {"Kagolix": KagolixConfig, "Sisavik": SisavikConfig, "Gizezen": GizezenConfig}
 
 
 def load_config(model_path: str):

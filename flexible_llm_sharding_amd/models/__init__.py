@@ -11,4 +11,7 @@ def hybrid_family(cfg):
     if fam == "sisavik":
         from . import sisavik
         return sisavik
+    if fam == "gizezen":
+        from . import gizezen
+        return gizezen
     raise NotImplementedError(f"no hybrid family {fam!r}")

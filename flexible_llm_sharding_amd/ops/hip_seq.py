@@ -55,7 +55,7 @@ class HipSeqOps:
         self._freqs = {}
 
     # ----------------------------------------------------------------- rows
-    def embed_rows(self, ids, table, out=None):
+    def embed_rows(self, ids, table, out=None, scale=1.0):
         T, (V, D) = ids.numel(), table.shape
         if out is None:
             out = torch.empty(T, D, dtype=torch.float32, device=table.device)
@@ -63,7 +63,7 @@ class HipSeqOps:
             raise TypeError("embed_rows: out must be a contiguous fp32 [T, D] tensor")
         _vec(ids, "ids", T, torch.int32)
         _chk(self.k.fls_seq_embed(ids.data_ptr(), table.data_ptr(), _code(table, "table"), out.data_ptr(), T, D, V,
-                                  _stream()), "fls_seq_embed")
+                                  float(scale), _stream()), "fls_seq_embed")
         return out
 
     def group_rmsnorm(self, x, w, groups, eps, out_dtype, row_idx=None, w_offset=0.0):
@@ -88,6 +88,29 @@ class HipSeqOps:
         _chk(self.k.fls_seq_group_rmsnorm(y.data_ptr(), y.stride(0), None, w.data_ptr(), x.data_ptr(), 0, x.stride(0),
                                           x.shape[0], x.shape[1], groups, float(eps), 1, float(w_offset), _stream()),
              "fls_seq_group_rmsnorm")
+        return x
+
+    def dyt_norm(self, x, wb, alpha, out_dtype, row_idx=None):
+        _rows(x, "x", torch.float32)
+        rows = x.shape[0] if row_idx is None else row_idx.numel()
+        D = x.shape[1]
+        _vec(wb, "wb", 2 * D)
+        _vec(alpha, "alpha", 1)
+        if row_idx is not None:
+            _vec(row_idx, "row_idx", rows, torch.int32)
+        y = torch.empty(rows, D, dtype=out_dtype, device=x.device)
+        _chk(self.k.fls_seq_dyt_norm(x.data_ptr(), x.stride(0), row_idx.data_ptr() if row_idx is not None else None,
+                                     wb.data_ptr(), alpha.data_ptr(), y.data_ptr(), _CODE[out_dtype], D, rows, D, _stream()),
+             "fls_seq_dyt_norm")
+        return y
+
+    def add_scaled_(self, x, y, mult):
+        _rows(x, "x", torch.float32)
+        _rows(y, "y", torch.float32)
+        if x.shape != y.shape:
+            raise ValueError("add_scaled_: shapes differ")
+        _chk(self.k.fls_seq_add_scaled(x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0), x.shape[0], x.shape[1],
+                                       float(mult), _stream()), "fls_seq_add_scaled")
         return x
 
     def _gemm(self, a, w, c, bias, M, N, K, lda, ldw, ldc, groups=1, offs=None, a_gs=0, a_mod=1, w_gs=0, c_gs=0,
@@ -186,16 +209,15 @@ class HipSeqOps:
                    a_mod=heads, w_gs=N * K, c_gs=out_stride)
         return out
 
-    def rope_freqs(self, dims, base, device):
-        key = (int(dims), float(base), str(device))
+    def rope_freqs(self, dims, base, device, scaling=None):
+        key = (int(dims), float(base), str(device), None if scaling is None else tuple(float(v) for v in scaling))
         if key not in self._freqs:
-            i = torch.arange(dims // 2, dtype=torch.float64)
-            f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float()
-            self._freqs[key] = f.to(device)
+            from .torch_seq import TorchSeqOps
+            self._freqs[key] = TorchSeqOps.rope_freqs(int(dims), float(base), device, scaling)
         return self._freqs[key]
 
     def head_norm_rope(self, x, heads, n, x_col, x_hs, out, out_col, out_hs, meta, w=None, eps=0.0, rot=None,
-                       row_map=None, raw=None):
+                       row_map=None, raw=None, unit_after=False):
         _rows(x, "x")
         _rows(out, "out")
         T = x.shape[0]
@@ -213,14 +235,15 @@ class HipSeqOps:
         dims, freqs = 0, None
         if rot is not None and rot[0] > 0:
             dims = int(rot[0])
-            freqs = self.rope_freqs(dims, rot[1], x.device)
+            freqs = self.rope_freqs(dims, rot[1], x.device, rot[2] if len(rot) > 2 else None)
         _chk(self.k.fls_seq_head_norm_rope(x.data_ptr(), _code(x, "x"), x.stride(0), x_col, x_hs, heads, n,
                                            w.data_ptr() if w is not None else None, float(eps),
                                            freqs.data_ptr() if freqs is not None else None, dims, meta["tok_pos"].data_ptr(),
                                            row_map.data_ptr() if row_map is not None else None, out.data_ptr(),
                                            _code(out, "out"), out.stride(0), out_col, out_hs,
                                            raw.data_ptr() if raw is not None else None,
-                                           raw.stride(0) if raw is not None else 0, T, _stream()), "fls_seq_head_norm_rope")
+                                           raw.stride(0) if raw is not None else 0, T, 1 if unit_after else 0, _stream()),
+             "fls_seq_head_norm_rope")
         return out
 
     def softcap_(self, z, cap):
@@ -260,7 +283,7 @@ class HipSeqOps:
                                      kcols, vcols, _stream()), "fls_seq_kv_store")
 
     def attn_paged(self, q, kcache, vcache, meta, H, G, d, dv, scale, softcap, r1, r2, chunk, page_size, out_dtype,
-                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None):
+                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None, sink=None, head_gate=None):
         _rows(q, "q")
         T = q.shape[0]
         if kcache.dtype != out_dtype or vcache.dtype != out_dtype or q.shape[1] != H * d \
@@ -281,6 +304,14 @@ class HipSeqOps:
         elif out.dtype != out_dtype or tuple(out.shape) != (T, H * dv):
             raise TypeError("attn_paged: out does not fit")
         _rows(out, "out")
+        if head_gate is not None:
+            _rows(head_gate, "head_gate", torch.float32)
+            if tuple(head_gate.shape) != (T, H):
+                raise ValueError("attn_paged: head_gate is [T, H]")
+        if sink is not None and gate_bias is not None:
+            raise ValueError("attn_paged: a silent softmax entry and per-key sigmoid weights exclude each other")
+        extra = (1 if sink is not None else 0, float(sink or 0.0), head_gate.data_ptr() if head_gate is not None else None,
+                 head_gate.stride(0) if head_gate is not None else 0)
         tiles = meta.get("q_tiles")
         if tiles is not None and kcache.dtype == torch.bfloat16 and d in (64, 128) and dv in (64, 128):
             # a step with many rows per request: the matrix-core kernel over row tiles
@@ -291,7 +322,7 @@ class HipSeqOps:
                                              r1.data_ptr() if r1 is not None else None,
                                              r2.data_ptr() if r2 is not None else None, int(chunk), int(window),
                                              int(keep_first), gate_bias.data_ptr() if gate_bias is not None else None,
-                                             float(out_scale), int(page_size), _stream())
+                                             float(out_scale), int(page_size), *extra, _stream())
             if rc == 0:
                 return out
             if rc != -2:
@@ -302,7 +333,7 @@ class HipSeqOps:
         if window > 0:
             bound = min(bound, int(window) + int(keep_first))
         if tiles is None and q.dtype == torch.float32 and kcache.dtype == torch.bfloat16 and gate_bias is None and r1 is None \
-                and softcap == 0 and chunk == 0 and H // G <= 32 and (d, dv) in self.HEAD_TILE_SHAPES:
+                and sink is None and head_gate is None and softcap == 0 and chunk == 0 and H // G <= 32 and (d, dv) in self.HEAD_TILE_SHAPES:
             # few rows whose heads share long key / value rows (decoding over cached latent rows): the heads of a
             # token as the columns of one matrix-core tile, every key tile staged once for all of them
             ns = max(1, min(16, 256 // max(1, T * G), bound // 32))
@@ -326,8 +357,8 @@ class HipSeqOps:
                                        float(scale), float(softcap), r1.data_ptr() if r1 is not None else None,
                                        r2.data_ptr() if r2 is not None else None, int(chunk), int(window), int(keep_first),
                                        gate_bias.data_ptr() if gate_bias is not None else None, float(out_scale),
-                                       int(page_size), nsplit, part.data_ptr() if part is not None else None, _stream()),
-             "fls_seq_attn_paged")
+                                       int(page_size), nsplit, part.data_ptr() if part is not None else None, *extra,
+                                       _stream()), "fls_seq_attn_paged")
         return out
 
     # ------------------------------------------------------------ recurrences
@@ -422,10 +453,39 @@ class HipSeqOps:
         return out
 
     # ------------------------------------------------------ mixture of experts
+    def moe_route_topk(self, logits, top):
+        """The ``top`` largest logits choose; the softmax over the chosen logits weighs."""
+        return self.moe_route_corrected(logits, None, top)
+
+    def moe_combine_(self, x, y, route, mult, shared=None, shared_gate=None):
+        _rows(x, "x", torch.float32)
+        _rows(y, "y", torch.float32)
+        T, top = route.dest.shape
+        D = x.shape[1]
+        if x.shape[0] != T or y.shape[1] != D:
+            raise ValueError("moe_combine_: shapes do not fit")
+        if shared is not None:
+            _rows(shared, "shared", torch.float32)
+            if tuple(shared.shape) != (T, D):
+                raise ValueError("moe_combine_: the shared expert's rows do not fit")
+            if shared_gate is not None:
+                _rows(shared_gate, "shared_gate", torch.float32)
+                if tuple(shared_gate.shape) != (T, 1):
+                    raise ValueError("moe_combine_: shared_gate is [T, 1]")
+        _chk(self.k.fls_seq_moe_combine(x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0), route.dest.data_ptr(),
+                                        route.w.data_ptr(), T, top, shared.data_ptr() if shared is not None else None,
+                                        shared.stride(0) if shared is not None else 0,
+                                        shared_gate.data_ptr() if shared is not None and shared_gate is not None else None,
+                                        shared_gate.stride(0) if shared is not None and shared_gate is not None else 0, D,
+                                        float(mult), _stream()), "fls_seq_moe_combine")
+        return x
+
     def moe_route_corrected(self, logits, corr, top):
+        """``corr`` None: top-k on the bare logits, softmax over the chosen."""
         _rows(logits, "logits", torch.float32)
         T, E = logits.shape
-        _vec(corr, "corr", E)
+        if corr is not None:
+            _vec(corr, "corr", E)
         dev = logits.device
         ids = torch.empty(T, top, dtype=torch.int32, device=dev)
         w = torch.empty(T, top, dtype=torch.float32, device=dev)
@@ -434,7 +494,7 @@ class HipSeqOps:
         dest = torch.empty(T, top, dtype=torch.int32, device=dev)
         rows = torch.empty(T * top, dtype=torch.int32, device=dev)
         s = _stream()
-        _chk(self.k.fls_seq_moe_route(logits.data_ptr(), logits.stride(0), corr.data_ptr(), T, E, top, ids.data_ptr(),
+        _chk(self.k.fls_seq_moe_route(logits.data_ptr(), logits.stride(0), corr.data_ptr() if corr is not None else None, T, E, top, ids.data_ptr(),
                                       w.data_ptr(), hist.data_ptr(), s), "fls_seq_moe_route")
         _chk(self.k.fls_seq_moe_scan(hist.data_ptr(), E, offs.data_ptr(), cursor.data_ptr(), s), "fls_seq_moe_scan")
         _chk(self.k.fls_seq_moe_place(ids.data_ptr(), T * top, top, cursor.data_ptr(), dest.data_ptr(), rows.data_ptr(), s),

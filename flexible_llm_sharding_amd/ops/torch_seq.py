@@ -28,8 +28,10 @@ class SeqRoute:
 
 class TorchSeqOps:
     # ----------------------------------------------------------------- rows
-    def embed_rows(self, ids, table, out=None):
+    def embed_rows(self, ids, table, out=None, scale=1.0):
         e = table.index_select(0, ids.long()).float()
+        if scale != 1.0:
+            e = e * scale
         if out is not None:
             out.copy_(e)
             return out
@@ -46,6 +48,18 @@ class TorchSeqOps:
 
     def add_group_rmsnorm_(self, x, y, w, groups, eps, w_offset=0.0):
         x.add_(self.group_rmsnorm(y, w, groups, eps, torch.float32, w_offset=w_offset))
+        return x
+
+    def dyt_norm(self, x, wb, alpha, out_dtype, row_idx=None):
+        """Dynamic Tanh: tanh(alpha x) w + b elementwise, no statistics of the row; ``wb`` = [w; b] ([2, D]),
+        ``alpha`` a one-element tensor."""
+        if row_idx is not None:
+            x = x.index_select(0, row_idx.long())
+        return (torch.tanh(alpha.float() * x.float()) * wb[0].float() + wb[1].float()).to(out_dtype)
+
+    def add_scaled_(self, x, y, mult):
+        """x += mult * y (the residual update of a sublayer whose output joins the stream scaled)."""
+        x.add_(y.float(), alpha=float(mult))
         return x
 
     def matmul_nt(self, a, w, bias=None, xielu=None, out_dtype=torch.float32):
@@ -111,31 +125,46 @@ class TorchSeqOps:
         return out
 
     @staticmethod
-    def rope_freqs(dims, base, device):
-        """f_i = base^(-2i / dims), i < dims / 2, rounded once to fp32."""
+    def rope_freqs(dims, base, device, scaling=None):
+        """f_i = base^(-2i / dims), i < dims / 2, rounded once to fp32.  ``scaling`` = (factor, low, high,
+        original): a frequency whose wavelength 2 pi / f is longer than original / low is divided by
+        factor, one shorter than original / high stays, and between them the two are blended linearly in
+        s = (original / wavelength - low) / (high - low)."""
         i = torch.arange(dims // 2, dtype=torch.float64)
-        return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float().to(device)
+        f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
+        if scaling is not None:
+            factor, low, high, orig = (float(v) for v in scaling)
+            wl = 2 * math.pi / f
+            s_ = (orig / wl - low) / (high - low) if high != low else torch.ones_like(f)
+            mid = (1 - s_) * f / factor + s_ * f
+            f = torch.where(wl < orig / high, f, torch.where(wl > orig / low, f / factor, mid))
+        return f.float().to(device)
 
     def head_norm_rope(self, x, heads, n, x_col, x_hs, out, out_col, out_hs, meta, w=None, eps=0.0, rot=None,
-                       row_map=None, raw=None):
+                       row_map=None, raw=None, unit_after=False):
         """Per row t and head h the n entries x[t, x_col + h * x_hs : + n]: RMS-normed over n times w
-        (when w is given), then the first rot = (dims, base)[0] entries rotated in pairs (2i, 2i + 1) by
-        the angle pos_t * base^(-2i / dims); written to out[row, out_col + h * out_hs : + n], row = t or
-        row_map[t].  ``raw``: a matrix like out that receives the entries as they came."""
+        (when w is given), then the first rot = (dims, base[, scaling])[0] entries rotated in pairs
+        (2i, 2i + 1) by the angle pos_t * f_i (``rope_freqs``), then, with ``unit_after``, divided by
+        their root mean square over n (eps inside the root, no weight); written to
+        out[row, out_col + h * out_hs : + n], row = t or row_map[t].  ``raw``: a matrix like out that
+        receives the entries as they came."""
         T = x.shape[0]
         v = torch.stack([x[:, x_col + h * x_hs:x_col + h * x_hs + n] for h in range(heads)], 1).float()    # [T, heads, n]
         keep = v.clone()
         if w is not None:
             v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()
         if rot is not None and rot[0] > 0:
-            dims, base = rot
-            ang = meta["tok_pos"].float()[:, None] * self.rope_freqs(dims, base, x.device)[None, :]    # fp32 angles
+            dims, base = rot[0], rot[1]
+            freqs = self.rope_freqs(dims, base, x.device, rot[2] if len(rot) > 2 else None)
+            ang = meta["tok_pos"].float()[:, None] * freqs[None, :]                                     # fp32 angles
             c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
             a, b = v[:, :, 0:dims:2], v[:, :, 1:dims:2]
             r = v.clone()
             r[:, :, 0:dims:2] = a * c - b * s_
             r[:, :, 1:dims:2] = b * c + a * s_
             v = r
+        if unit_after:
+            v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
         rows = row_map.long() if row_map is not None else torch.arange(T, device=x.device)
         for h in range(heads):
             out[rows, out_col + h * out_hs:out_col + h * out_hs + n] = v[:, h].to(out.dtype)
@@ -159,13 +188,15 @@ class TorchSeqOps:
         vcache.view(-1, vcache.shape[-1]).index_copy_(0, kv_slot.long(), v.to(vcache.dtype))
 
     def attn_paged(self, q, kcache, vcache, meta, H, G, d, dv, scale, softcap, r1, r2, chunk, page_size, out_dtype,
-                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None):
+                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None, sink=None, head_gate=None):
         """Row i of a request sees the keys j <= i of its own chunk (``chunk`` > 0: floor(i / chunk) ==
         floor(j / chunk)) or window (``window`` > 0: j > i - window, and besides them the first
         ``keep_first`` keys of the sequence), read from the request's pages.  Head h of H reads key /
         value head h // (H / G): the first G * d (G * dv) columns of a pool row.  Weights: softmax over
         the visible keys of cap(scale q.k) - r1 log(1 + r2 (i - j)), or, with ``gate_bias`` [H],
-        sigmoid(scale q.k + gate_bias[h]) for each key by itself.  The result times ``out_scale``."""
+        sigmoid(scale q.k + gate_bias[h]) for each key by itself.  ``sink`` (a number): the softmax has one
+        more entry of that score and no value, p_j = exp(s_j) / (exp(sink) + sum exp(s)).  ``head_gate``
+        [T, H] fp32: head h's output of row t times sigmoid(head_gate[t, h]).  The result times ``out_scale``."""
         T = q.shape[0]
         res = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
         kf = kcache.reshape(-1, kcache.shape[-1])[:, :G * d].reshape(-1, G, d)
@@ -188,8 +219,16 @@ class TorchSeqOps:
                 s = softcap * torch.tanh(s / softcap)
             if r1 is not None:
                 s = s - r1.float()[:, None] * torch.log1p(r2.float()[:, None] * (i - js).float()[None, :])
-            p = torch.softmax(s, -1) if gate_bias is None else torch.sigmoid(s + gate_bias.float()[:, None])
-            res[t] = torch.einsum("hn,nhv->hv", p, vv.repeat_interleave(rep, 1)).reshape(-1) * out_scale
+            if gate_bias is not None:
+                p = torch.sigmoid(s + gate_bias.float()[:, None])
+            elif sink is not None:
+                p = torch.softmax(torch.cat([s, torch.full((H, 1), float(sink), device=q.device)], -1), -1)[:, :-1]
+            else:
+                p = torch.softmax(s, -1)
+            o = torch.einsum("hn,nhv->hv", p, vv.repeat_interleave(rep, 1))
+            if head_gate is not None:
+                o = o * torch.sigmoid(head_gate[t].float())[:, None]
+            res[t] = o.reshape(-1) * out_scale
         if out is not None:
             out.copy_(res.to(out.dtype))
             return out
@@ -302,6 +341,20 @@ class TorchSeqOps:
         offs[1:] = torch.cumsum(torch.bincount(flat, minlength=E), 0)
         return SeqRoute(ids.int(), w, offs, (order // top).int(), dest.int().reshape(T, top), top)
 
+    def moe_route_topk(self, logits, top):
+        """The ``top`` largest logits are chosen (ties: the lower expert), weighted by the softmax over
+        the chosen logits only."""
+        T, E = logits.shape
+        vals, ids = torch.sort(logits.float(), dim=-1, descending=True, stable=True)
+        ids, w = ids[:, :top], torch.softmax(vals[:, :top], -1)
+        flat = ids.reshape(-1)
+        order = torch.sort(flat, stable=True).indices
+        dest = torch.empty_like(order)
+        dest[order] = torch.arange(order.numel(), device=order.device)
+        offs = torch.zeros(E + 1, dtype=torch.int32, device=logits.device)
+        offs[1:] = torch.cumsum(torch.bincount(flat, minlength=E), 0)
+        return SeqRoute(ids.int(), w, offs, (order // top).int(), dest.int().reshape(T, top), top)
+
     def grouped_matmul_nt(self, a, w, offs):
         E, N, K = w.shape
         out = torch.zeros(a.shape[0], N, dtype=torch.float32, device=a.device)
@@ -314,6 +367,17 @@ class TorchSeqOps:
     def moe_weighted_sum(self, y, route):
         T, top = route.dest.shape
         return (y[route.dest.long().reshape(-1)].reshape(T, top, -1) * route.w[:, :, None]).sum(1)
+
+    def moe_combine_(self, x, y, route, mult, shared=None, shared_gate=None):
+        """x += mult * (sum_k w[t, k] y[dest[t, k]] + sigmoid(shared_gate[t]) * shared[t]): the experts'
+        weighted sum, the gated shared expert (both optional parts fp32; ``shared_gate`` [T, 1]) and the
+        residual update in one pass."""
+        s = self.moe_weighted_sum(y, route)
+        if shared is not None:
+            g = torch.sigmoid(shared_gate.float()) if shared_gate is not None else 1.0
+            s = s + g * shared.float()
+        x.add_(s, alpha=float(mult))
+        return x
 
     def argmax_f32(self, z):
         return z.argmax(-1).int()
