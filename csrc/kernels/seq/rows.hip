@@ -381,8 +381,9 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int ldl, cons
       chosen[k] = be;
       val[k] = best;
     }
-    float sum = 0.f;                                  // val[0] is the largest
-    for (int k = 0; k < top; ++k) { val[k] = expf(val[k] - val[0]); sum += val[k]; }
+    const float mx = val[0];                          // (the first choice is the largest)
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) { val[k] = expf(val[k] - mx); sum += val[k]; }
     const float inv = 1.f / sum;
     for (int k = 0; k < top; ++k) {
       ids[(size_t)t * top + k] = chosen[k];

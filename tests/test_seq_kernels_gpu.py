@@ -368,3 +368,121 @@ def test_heads_of_a_token_share_one_matrix_core_tile(ops, d, dv, Hh):
         kw = dict(scale=d ** -0.5, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, window=window,
                   keep_first=keep, out_scale=0.9)
         close(H.attn_paged(q, pool, pool, md, Hh, 1, d, dv, **kw), R.attn_paged(q, pool, pool, md, Hh, 1, d, dv, **kw), 2e-2)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+def test_dyt_norm_scaled_add_and_embedding_scale(ops, cdt, tol):
+    """Dynamic Tanh norm (vector path and odd widths, row gather, column slices), x += m y, embedding rows times a scale."""
+    H, R = ops
+    torch.manual_seed(11)
+    for T, D in ((7, 320), (3, 37), (130, 2048), (1, 4100)):
+        x = torch.randn(T, D + 8, device=DEV)[:, 4:4 + D] * 2
+        wb = torch.randn(2, D, device=DEV)
+        alpha = torch.tensor([0.7], device=DEV)
+        close(H.dyt_norm(x, wb, alpha, cdt), R.dyt_norm(x, wb, alpha, cdt), tol)
+        xc = x.contiguous()
+        close(H.dyt_norm(xc, wb, alpha, cdt), R.dyt_norm(xc, wb, alpha, cdt), tol)
+        idx = torch.tensor([T - 1, 0, T // 2], dtype=torch.int32, device=DEV)
+        close(H.dyt_norm(xc, wb, alpha, torch.float32, row_idx=idx), R.dyt_norm(xc, wb, alpha, torch.float32, row_idx=idx), 1e-5)
+        y = torch.randn(T, D, device=DEV)
+        a, b = xc.clone(), xc.clone()
+        close(H.add_scaled_(a, y, 0.6), R.add_scaled_(b, y, 0.6), 1e-6)
+        ys = torch.randn(T, D + 3, device=DEV)[:, 1:1 + D]
+        close(H.add_scaled_(a, ys, -1.3), R.add_scaled_(b, ys, -1.3), 1e-6)
+    table = torch.randn(50, 36, device=DEV).to(cdt)
+    ids = torch.tensor([3, 49, 0, 3], dtype=torch.int32, device=DEV)
+    close(H.embed_rows(ids, table, scale=0.37), R.embed_rows(ids, table, scale=0.37), 1e-6)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+def test_rotation_with_rescaled_frequencies_then_unit_norm(ops, cdt, tol):
+    """Pair rotation with wavelength-rescaled frequencies followed by the weightless RMS norm, into rows and into pools;
+    a plain placement (no norm, no rotation) of value heads."""
+    H, R = ops
+    torch.manual_seed(12)
+    lens, pos0 = [1, 40, 3, 130], [900, 0, 17, 2000]
+    md, n_pages, _ = meta_of(lens, pos0, DEV)
+    T = sum(lens)
+    sc = (8.0, 1.0, 4.0, 64)
+    f = R.rope_freqs(16, 100.0, "cpu", sc).double()
+    f0 = R.rope_freqs(16, 100.0, "cpu").double()
+    ratio = (f / f0).numpy()
+    assert ratio[0] == 1.0 and abs(ratio[-1] - 1 / 8) < 1e-6 and ((ratio[1:] <= ratio[:-1] + 1e-9).all())   # kept, blended, slowed
+    assert ((ratio > 1 / 8 + 1e-3) & (ratio < 1 - 1e-3)).any()
+    for heads, n, x_col, rot in ((3, 24, 5, (16, 100.0, sc)), (2, 40, 0, (40, 30000.0, (4.0, 2.0, 8.0, 512))), (4, 64, 0, (32, 1e4, None)),
+                                 (1, 6, 2, None), (2, 130, 0, (128, 500.0, None))):
+        x = torch.randn(T, x_col + heads * n + 3, device=DEV) * 3
+        for paged in (False, True):
+            rows = n_pages * 16 if paged else T
+            outs = []
+            for O in (H, R):
+                out = torch.zeros(rows, heads * n, device=DEV, dtype=cdt)
+                O.head_norm_rope(x, heads, n, x_col, n, out, 0, n, md, eps=1e-5, rot=rot, unit_after=True,
+                                 row_map=md["kv_slot"] if paged else None)
+                outs.append(out)
+            close(outs[0], outs[1], max(tol, 3e-4))
+            if not paged:                                       # every head has unit mean square
+                ms = outs[0].float().view(T, heads, n).pow(2).mean(-1)
+                assert (ms - 1).abs().max().item() < (2e-2 if cdt == torch.bfloat16 else 1e-3)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("Hh,G,d,dv", [(5, 5, 40, 72), (6, 2, 24, 40), (4, 2, 64, 64), (8, 2, 128, 128), (4, 4, 128, 64), (3, 1, 20, 14)])
+def test_attention_with_a_silent_softmax_entry_and_head_gates(ops, cdt, tol, Hh, G, d, dv):
+    """Windowed softmax with one more entry of a given score and no value, and a sigmoid gate per (row, head): prompts
+    (per-row kernel, and row tiles on the matrix cores where the head sizes allow), portions, decode rows."""
+    H, R = ops
+    torch.manual_seed(13)
+    lens, pos0 = [1, 170, 2, 33, 1], [150, 0, 64, 31, 3]
+    md, n_pages, _ = meta_of(lens, pos0, DEV)
+    T = sum(lens)
+    kc = (torch.randn(n_pages, 16, G * d, device=DEV) * 0.5).to(cdt)
+    vc = torch.randn(n_pages, 16, G * dv, device=DEV).to(cdt)
+    z = torch.randn(T, Hh * d + Hh + 5, device=DEV)
+    hg = z[:, Hh * d:Hh * d + Hh]                               # a column block of a wider matrix
+    q = torch.randn(T, Hh * d, device=DEV) * (8 / d) ** 0.5      # (scores of a few units whatever the head size)
+    for window, sink, gate, scale in ((9, 0.0, hg, 0.2), (72, 0.0, hg, 0.5), (72, 1.5, None, 0.2), (1, 0.0, hg, 0.3), (0, -2.0, hg, 0.05),
+                                      (40, None, hg, 0.2), (40, 0.0, hg, 1.5), (40, 0.0, hg, -1.5)):
+        kw = dict(scale=scale, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, window=window, sink=sink,
+                  head_gate=gate)
+        a = H.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw)
+        b = R.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw)
+        close(a, b, tol)
+    # decode rows far into their sequences: every row's keys cut over blocks, the silent entry joins once in the merge
+    lens, pos0 = [1, 1, 1], [1500, 3, 700]
+    md, n_pages, _ = meta_of(lens, pos0, DEV)
+    kc = (torch.randn(n_pages, 16, G * d, device=DEV) * 0.5).to(cdt)
+    vc = torch.randn(n_pages, 16, G * dv, device=DEV).to(cdt)
+    q = torch.randn(3, Hh * d, device=DEV) * (8 / d) ** 0.5
+    hg = torch.randn(3, Hh, device=DEV)
+    for window, sink, scale in ((0, 0.0, 0.3), (1000, 0.0, 0.01), (1000, 3.0, 0.3), (600, 0.0, -1.0)):
+        kw = dict(scale=scale, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, window=window, sink=sink, head_gate=hg)
+        close(H.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw), R.attn_paged(q, kc, vc, md, Hh, G, d, dv, **kw), tol)
+
+
+@pytest.mark.parametrize("T,E,top", [(33, 10, 3), (700, 8, 2), (5, 40, 9), (300, 3, 1), (4, 8, 8), (1, 5, 5)])
+def test_topk_routing_and_combine(ops, T, E, top):
+    """The largest logits choose, the softmax over the chosen weighs; the combine adds the weighted expert rows, the gated
+    shared expert's row and the residual in one pass."""
+    H, R = ops
+    torch.manual_seed(14)
+    D = 52
+    z = torch.randn(T, E + 3, device=DEV)
+    logits = z[:, 1:1 + E]
+    a, b = H.moe_route_topk(logits, top), R.moe_route_topk(logits, top)
+    assert torch.equal(a.ids.cpu().long(), b.ids.cpu().long())
+    close(a.w, b.w, 1e-5)
+    assert (a.w.sum(-1) - 1).abs().max().item() < 1e-5
+    assert torch.equal(a.offs.cpu().long(), b.offs.cpu().long())
+    # a tie goes to the lower expert
+    tie = torch.zeros(2, E, device=DEV)
+    assert H.moe_route_topk(tie, top).ids.cpu().tolist() == [list(range(top))] * 2
+    y = torch.randn(T * top, D, device=DEV)
+    shared = torch.randn(T, D, device=DEV)
+    gate = torch.randn(T, 4, device=DEV)[:, 2:3]
+    for sh, g in ((None, None), (shared, gate), (shared, None)):
+        x1, x2 = torch.randn(T, D, device=DEV), None
+        x2 = x1.clone()
+        H.moe_combine_(x1, y, a, 0.6, sh, g)
+        R.moe_combine_(x2, y, a, 0.6, sh, g)
+        close(x1, x2, 1e-5)
