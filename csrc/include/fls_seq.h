@@ -30,6 +30,9 @@ int fls_seq_embed(const int* ids, const void* table, int tt, float* out, int T, 
 // Dynamic Tanh norm: y[r, c] = tanh(alpha[0] x[row, c]) wb[c] + wb[D + c], row = idx ? idx[r] : r; y of type ty
 int fls_seq_dyt_norm(const float* x, int ldx, const int* idx, const float* wb, const float* alpha, void* y, int ty,
                      int ldy, int rows, int D, fls_stream_t s);
+// x += mult * y, then h = tanh(alpha[0] x) wb[c] + wb[D + c] of the new x (h of type th): residual update + next norm
+int fls_seq_add_scaled_dyt(float* x, int ldx, const float* y, int ldy, float mult, const float* wb, const float* alpha,
+                           void* h, int th, int ldh, int rows, int D, fls_stream_t s);
 // x += mult * y (fp32 rows)
 int fls_seq_add_scaled(float* x, int ldx, const float* y, int ldy, int rows, int D, float mult, fls_stream_t s);
 int fls_seq_gather_rows(const void* x, int tx, int ldx, const int* idx, void* y, int ldy, int rows, int D, fls_stream_t s);
@@ -91,6 +94,14 @@ int fls_seq_attn_heads(const void* q, int ldq, const void* kc, int ldk, const vo
 int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b, float* state, void* out, int to, int ldo,
                         const int* tok_seq, const int* cu, const int* pos0, const int* slot, int T, int B, int C,
                         int taps, int act, int residual, int one_row_each, fls_stream_t s);
+// projected rows z = [q (H d) | k (G d) | v (G dv) | ...] into attention in one pass: causal convolution per channel
+// (w [C, taps] nullable, history in state[slot][taps-1][C] as for fls_seq_causal_conv), q and k heads rotated in pairs
+// over their first rot entries (angle tok_pos * freqs[i]) and divided by sqrt(mean(head^2) + eps), q to qo (fp32
+// [T, H d]), k and v (v as convolved) to row kv_slot[t] of pools of type tc.  G = 0: queries only.  d, dv <= 512
+int fls_seq_qkv_conv_rope(const float* z, int ldz, const float* w, float* state, int taps, const int* tok_seq,
+                          const int* tok_pos, const int* cu, const int* pos0, const int* slot, const int* kv_slot,
+                          int T, int B, int H, int G, int d, int dv, float eps, const float* freqs, int rot, float* qo,
+                          int ldq, void* kc, int ldk, void* vc, int ldv, int tc, int one_row_each, fls_stream_t s);
 // generalized delta rule, per head a state S[d][d] in state[slot][H][d][d]:
 // S_t = diag(w) S_(t-1) - (a * u)(u^T S_(t-1)) + k v^T, o = S_t^T r; u = k / sqrt(sum k^2 + key_eps),
 // w = exp(-decay_scale sigmoid(wz + w0)), a = sigmoid(az); out = out_scale o / rms_head(o; norm_eps) norm_w sigmoid(g).

@@ -109,6 +109,57 @@ extern "C" int fls_seq_add_scaled(float* x, int ldx, const float* y, int ldy, in
   return 0;
 }
 
+// x[r, c] += mult * y[r, c] and h[r, c] = tanh(alpha x[r, c]) w[c] + b[c] of the new x: the residual update and the
+// next sublayer's Dynamic Tanh norm in one pass over the stream
+template <typename TO>
+__global__ __launch_bounds__(256) void add_scaled_dyt_kernel(float* __restrict__ x, int ldx, const float* __restrict__ y, int ldy,
+                                                             float mult, const float* __restrict__ wb,
+                                                             const float* __restrict__ alpha, TO* __restrict__ h, int ldh,
+                                                             int D, int vec) {
+  const float a = alpha[0];
+  float* xr = x + (size_t)blockIdx.x * ldx;
+  const float* yr = y + (size_t)blockIdx.x * ldy;
+  TO* hr = h + (size_t)blockIdx.x * ldh;
+  const float* w = wb;
+  const float* b = wb + D;
+  const int c0 = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c0 >= D) return;
+  if (vec) {
+    float4 v = *reinterpret_cast<const float4*>(xr + c0);
+    const float4 u = *reinterpret_cast<const float4*>(yr + c0);
+    v.x += mult * u.x; v.y += mult * u.y; v.z += mult * u.z; v.w += mult * u.w;
+    *reinterpret_cast<float4*>(xr + c0) = v;
+    const float4 wv = *reinterpret_cast<const float4*>(w + c0), bv = *reinterpret_cast<const float4*>(b + c0);
+    const float o0 = tanhf(a * v.x) * wv.x + bv.x, o1 = tanhf(a * v.y) * wv.y + bv.y;
+    const float o2 = tanhf(a * v.z) * wv.z + bv.z, o3 = tanhf(a * v.w) * wv.w + bv.w;
+    if constexpr (sizeof(TO) == 2) {
+      bf16_t e[4] = {f_to_bf16(o0), f_to_bf16(o1), f_to_bf16(o2), f_to_bf16(o3)};
+      *reinterpret_cast<uint2*>(hr + c0) = *reinterpret_cast<const uint2*>(e);
+    } else {
+      *reinterpret_cast<float4*>(hr + c0) = make_float4(o0, o1, o2, o3);
+    }
+  } else {
+    for (int c = c0; c < min(D, c0 + 4); ++c) {
+      const float v = xr[c] + mult * yr[c];
+      xr[c] = v;
+      stf(hr, c, tanhf(a * v) * w[c] + b[c]);
+    }
+  }
+}
+
+extern "C" int fls_seq_add_scaled_dyt(float* x, int ldx, const float* y, int ldy, float mult, const float* wb, const float* alpha,
+                                      void* h, int th, int ldh, int rows, int D, fls_stream_t s) {
+  if (rows <= 0) return 0;
+  const int vec = D % 4 == 0 && ldx % 4 == 0 && ldy % 4 == 0 && ldh % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0 &&
+                  (uintptr_t)wb % 16 == 0 && (uintptr_t)h % 16 == 0;
+  dim3 grid(rows, (D + 1023) / 1024);
+  hipStream_t st = (hipStream_t)s;
+  if (th == 1) hipLaunchKernelGGL((add_scaled_dyt_kernel<bf16_t>), grid, dim3(256), 0, st, x, ldx, y, ldy, mult, wb, alpha, (bf16_t*)h, ldh, D, vec);
+  else hipLaunchKernelGGL((add_scaled_dyt_kernel<float>), grid, dim3(256), 0, st, x, ldx, y, ldy, mult, wb, alpha, (float*)h, ldh, D, vec);
+  SEQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ------------------------------------------------------------------------------- embedding
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int D, int V, float scale) {
@@ -525,4 +576,4 @@ extern "C" int fls_seq_moe_combine(float* x, int ldx, const float* y, int ldy, c
   return 0;
 }
 
-extern "C" int fls_seq_version(void) { return 8; }
+extern "C" int fls_seq_version(void) { return 9; }

@@ -136,6 +136,115 @@ extern "C" int fls_seq_causal_conv(const float* x, int ldx, const float* w, cons
   return 0;
 }
 
+// ------------------------------------------------ projected q | k | v rows on their way into attention
+// z = [q (H d) | k (G d) | v (G dv) | ...] per row.  One wave per (row, head of q, k or v): the head's entries pass the
+// causal convolution over the request's rows (w [C, taps], history from state[slot] as above; w null: none), then
+// -- q and k heads -- the rotation of pairs (2i, 2i + 1) of the first `rot` entries by the angle pos * freqs[i]
+// (the pair's other entry sits in the neighbouring lane) and the division by the head's root mean square (eps
+// inside the root); q goes to qo[t] (fp32), k and v to row kv_slot[t] of their pools.  fuse_state (every request
+// brings one row): the wave also rewrites its channels of the carried history.  Head sizes <= 512.
+#define QKV_MAX_E 8
+template <typename TO>
+__global__ __launch_bounds__(256) void qkv_conv_rope_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ w,
+                                                            float* __restrict__ state, int taps, const int* __restrict__ tok_seq,
+                                                            const int* __restrict__ tok_pos, const int* __restrict__ cu,
+                                                            const int* __restrict__ pos0, const int* __restrict__ slot,
+                                                            const int* __restrict__ kv_slot, int H, int G, int d, int dv, float eps,
+                                                            const float* __restrict__ freqs, int rot, float* __restrict__ qo,
+                                                            int ldq, TO* __restrict__ kc, int ldk, TO* __restrict__ vc, int ldv,
+                                                            int items, int C, int fuse_state) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= items) return;
+  const int ipr = H + 2 * G;
+  const int t = item / ipr, hi = item % ipr;
+  const int kind = hi < H ? 0 : (hi < H + G ? 1 : 2);
+  const int n = kind == 2 ? dv : d;
+  const int col0 = kind == 0 ? hi * d : (kind == 1 ? H * d + (hi - H) * d : (H + G) * d + (hi - H - G) * dv);
+  const int s = tok_seq[t];
+  const int tl = t - cu[s];
+  const bool carried = pos0[s] > 0;
+  float* hist = (w != nullptr && taps > 1) ? state + (size_t)slot[s] * (taps - 1) * C : nullptr;
+  float v[QKV_MAX_E];
+#pragma unroll
+  for (int e = 0; e < QKV_MAX_E; ++e) {
+    const int c = lane + 64 * e;
+    float acc = 0.f;
+    if (c < n) {
+      const int ch = col0 + c;
+      if (w == nullptr) {
+        acc = z[(size_t)t * ldz + ch];
+      } else {
+        for (int j = 0; j < taps; ++j) {
+          const int src = tl - j;
+          float in = 0.f;
+          if (src >= 0) in = z[(size_t)(t - j) * ldz + ch];
+          else if (carried) in = hist[(size_t)(taps - 1 + src) * C + ch];
+          acc += w[(size_t)ch * taps + (taps - 1 - j)] * in;
+        }
+        if (fuse_state && taps > 1) {                // the request's only row: shift the history, append this row
+          for (int k = 0; k + 2 < taps; ++k) hist[(size_t)k * C + ch] = carried ? hist[(size_t)(k + 1) * C + ch] : 0.f;
+          hist[(size_t)(taps - 2) * C + ch] = z[(size_t)t * ldz + ch];
+        }
+      }
+    }
+    v[e] = acc;
+  }
+  if (kind == 2) {
+    TO* vr = vc + (size_t)kv_slot[t] * ldv + (size_t)(hi - H - G) * dv;
+#pragma unroll
+    for (int e = 0; e < QKV_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) stf(vr, c, v[e]); }
+    return;
+  }
+  const float pos = rot > 0 ? (float)tok_pos[t] : 0.f;
+  float s2 = 0.f;
+#pragma unroll
+  for (int e = 0; e < QKV_MAX_E; ++e) {
+    const int c = lane + 64 * e;
+    const float other = __shfl_xor(v[e], 1, 64);
+    if (c < rot) {
+      const float ang = pos * freqs[c >> 1];
+      const float cs = cosf(ang), sn = sinf(ang);
+      v[e] = (c & 1) ? v[e] * cs + other * sn : v[e] * cs - other * sn;
+    }
+    s2 += v[e] * v[e];                                // (entries past n are zeros)
+  }
+  const float rs = 1.f / sqrtf(wave_sum(s2) / (float)n + eps);
+  if (kind == 0) {
+    float* qr = qo + (size_t)t * ldq + (size_t)hi * d;
+#pragma unroll
+    for (int e = 0; e < QKV_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) qr[c] = v[e] * rs; }
+  } else {
+    TO* kr = kc + (size_t)kv_slot[t] * ldk + (size_t)(hi - H) * d;
+#pragma unroll
+    for (int e = 0; e < QKV_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) stf(kr, c, v[e] * rs); }
+  }
+}
+
+extern "C" int fls_seq_qkv_conv_rope(const float* z, int ldz, const float* w, float* state, int taps, const int* tok_seq,
+                                     const int* tok_pos, const int* cu, const int* pos0, const int* slot, const int* kv_slot,
+                                     int T, int B, int H, int G, int d, int dv, float eps, const float* freqs, int rot, float* qo,
+                                     int ldq, void* kc, int ldk, void* vc, int ldv, int tc, int one_row_each, fls_stream_t s) {
+  if (T <= 0) return 0;
+  if (H < 1 || G < 0 || d < 1 || d > 64 * QKV_MAX_E || dv > 64 * QKV_MAX_E || rot < 0 || rot > d || (rot & 1) ||
+      (rot > 0 && freqs == nullptr) || (G > 0 && (kc == nullptr || vc == nullptr || kv_slot == nullptr || dv < 1)) ||
+      (w != nullptr && (taps < 1 || (taps > 1 && state == nullptr))))
+    return -1;
+  const int C = H * d + G * (d + dv);
+  if (C > ldz || H * d > ldq || (G > 0 && (G * d > ldk || G * dv > ldv))) return -1;
+  const int items = T * (H + 2 * G);
+  const int fuse = one_row_each && T == B;
+  hipStream_t st = (hipStream_t)s;
+  if (tc == 1) hipLaunchKernelGGL((qkv_conv_rope_kernel<bf16_t>), dim3((items + 3) / 4), dim3(256), 0, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (bf16_t*)kc, ldk, (bf16_t*)vc, ldv, items, C, fuse);
+  else hipLaunchKernelGGL((qkv_conv_rope_kernel<float>), dim3((items + 3) / 4), dim3(256), 0, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (float*)kc, ldk, (float*)vc, ldv, items, C, fuse);
+  SEQ_LAUNCH_CHECK();
+  if (w != nullptr && taps > 1 && !fuse) {
+    hipLaunchKernelGGL(conv_state_kernel, dim3((C + 255) / 256, B), dim3(256), 0, st, z, ldz, state, cu, pos0, slot, C, taps);
+    SEQ_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
 // ------------------------------------------------------------------- gated linear recurrence
 // one thread per (request, channel); sqrt(1 - a^2) from expm1 of the log decay, which keeps its
 // accuracy when a is close to 1

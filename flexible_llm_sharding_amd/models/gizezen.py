@@ -138,7 +138,7 @@ def state_spec(cfg) -> dict:
             paged[name] = {"k": m["kv_heads"] * m["dim"], "v": m["kv_heads"] * m["vdim"]}
         else:
             alias[name] = f"l{cfg.kv_owner(i)}"
-        if "conv" in m:
+        if _taps(m) > 1:
             slots[name] = {"conv": (_taps(m) - 1, sum(_cols(m)))}
         horizons.append(("window", _window(m) or NO_WINDOW, 0))
     return {"paged": paged, "alias": alias, "slots": slots, "horizons": horizons}
@@ -149,18 +149,14 @@ def _attention(ctx, m: dict, W, h, meta, name: str):
     ops, eps, cdt = ctx.ops, ctx.cfg.norm_eps, ctx.compute_dtype
     qs, ks, vs = _cols(m)
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    C, rot = qs + ks + vs, _rot(m)
+    C = qs + ks + vs
     z = ops.matmul_nt(h, W["win"])                                        # fp32 [T, q | k | v | g]
-    u = z[:, :C]
-    if "conv" in W:
-        u = ops.causal_conv(u, W["conv"], None, ctx.cache.recurrent(name)["conv"], meta)
     kc, vc = ctx.cache.kv(name)
     q = torch.empty(z.shape[0], qs, dtype=torch.float32, device=z.device)
-    ops.head_norm_rope(u, H, d, 0, d, q, 0, d, meta, eps=eps, rot=rot, unit_after=True)
-    if ks:
-        ops.head_norm_rope(u, G, d, qs, d, kc.view(-1, G * d), 0, d, meta, eps=eps, rot=rot, unit_after=True,
-                           row_map=meta["kv_slot"])
-        ops.head_norm_rope(u, G, dv, qs + ks, dv, vc.view(-1, G * dv), 0, dv, meta, row_map=meta["kv_slot"])
+    # convolution, rotation, unit norm and the write into the pages in one pass over the projected rows
+    st = ctx.cache.recurrent(name)["conv"] if "conv" in W and _taps(m) > 1 else None
+    ops.qkv_conv_rope_store(z, W.get("conv"), st, meta, H, G if ks else 0, d, dv, q, kc if ks else None, vc if ks else None,
+                            eps=eps, rot=_rot(m))
     a = ops.attn_paged(q, kc, vc, meta, H, G, d, dv, scale=float(m["scale"]), softcap=0.0, r1=None, r2=None, chunk=0,
                        page_size=ctx.cache.page_size, out_dtype=cdt, window=_window(m), sink=SINK_SCORE,
                        head_gate=z[:, C:C + H])
@@ -187,9 +183,11 @@ def run_block(ctx, W, x: torch.Tensor, meta: dict, name: str) -> torch.Tensor:
     cfg, ops, cdt = ctx.cfg, ctx.ops, ctx.compute_dtype
     L = cfg.layer(name)
     h = ops.dyt_norm(x, W["norm1"], W["alpha1"], cdt)
-    ops.add_scaled_(x, _attention(ctx, L.mixer, W, h, meta, name), cfg.residual_mult)
-    if L.mlp is not None:
-        _moe(ctx, L.mlp, W, ops.dyt_norm(x, W["norm2"], W["alpha2"], cdt), x)
+    y = _attention(ctx, L.mixer, W, h, meta, name)
+    if L.mlp is None:
+        return ops.add_scaled_(x, y, cfg.residual_mult)
+    # (the residual update and the feed-forward's norm read and write the stream once)
+    _moe(ctx, L.mlp, W, ops.add_scaled_dyt_norm_(x, y, cfg.residual_mult, W["norm2"], W["alpha2"], cdt), x)
     return x
 
 

@@ -113,6 +113,56 @@ class HipSeqOps:
                                        float(mult), _stream()), "fls_seq_add_scaled")
         return x
 
+    def add_scaled_dyt_norm_(self, x, y, mult, wb, alpha, out_dtype):
+        _rows(x, "x", torch.float32)
+        _rows(y, "y", torch.float32)
+        if x.shape != y.shape:
+            raise ValueError("add_scaled_dyt_norm_: shapes differ")
+        T, D = x.shape
+        _vec(wb, "wb", 2 * D)
+        _vec(alpha, "alpha", 1)
+        h = torch.empty(T, D, dtype=out_dtype, device=x.device)
+        _chk(self.k.fls_seq_add_scaled_dyt(x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0), float(mult), wb.data_ptr(),
+                                           alpha.data_ptr(), h.data_ptr(), _CODE[out_dtype], D, T, D, _stream()),
+             "fls_seq_add_scaled_dyt")
+        return h
+
+    def qkv_conv_rope_store(self, z, w, state, meta, H, G, d, dv, q_out, kc, vc, eps=0.0, rot=None):
+        _rows(z, "z", torch.float32)
+        _rows(q_out, "q_out", torch.float32)
+        T = z.shape[0]
+        C = H * d + G * (d + dv)
+        if z.shape[1] < C or tuple(q_out.shape) != (T, H * d):
+            raise ValueError("qkv_conv_rope_store: rows do not fit the head sizes")
+        taps = 1
+        if w is not None:
+            taps = w.shape[1]
+            _vec(w, "w", C * taps)
+            if taps > 1 and (state is None or state.dtype != torch.float32 or not state.is_contiguous()
+                             or tuple(state.shape[1:]) != (taps - 1, C)):
+                raise ValueError("qkv_conv_rope_store: state must be fp32 [slots, taps - 1, C]")
+        tc = 0
+        if G:
+            if kc.dtype != vc.dtype or kc.shape[-1] < G * d or vc.shape[-1] < G * dv or not kc.is_contiguous() \
+                    or not vc.is_contiguous():
+                raise ValueError("qkv_conv_rope_store: pools do not fit the head sizes")
+            tc = _code(kc, "kc")
+            _vec(meta["kv_slot"], "kv_slot", T, torch.int32)
+        dims, freqs = 0, None
+        if rot is not None and rot[0] > 0:
+            dims = int(rot[0])
+            freqs = self.rope_freqs(dims, rot[1], z.device, rot[2] if len(rot) > 2 else None)
+        _chk(self.k.fls_seq_qkv_conv_rope(z.data_ptr(), z.stride(0), w.data_ptr() if w is not None else None,
+                                          state.data_ptr() if state is not None and taps > 1 else None, taps,
+                                          meta["tok_seq"].data_ptr(), meta["tok_pos"].data_ptr(), meta["cu"].data_ptr(),
+                                          meta["pos0"].data_ptr(), meta["slot"].data_ptr(),
+                                          meta["kv_slot"].data_ptr() if G else None, T, meta["n_seqs"], H, G, d, dv, float(eps),
+                                          freqs.data_ptr() if freqs is not None else None, dims, q_out.data_ptr(),
+                                          q_out.stride(0), kc.data_ptr() if G else None, kc.shape[-1] if G else 0,
+                                          vc.data_ptr() if G else None, vc.shape[-1] if G else 0, tc,
+                                          1 if meta.get("max_rows") == 1 else 0, _stream()), "fls_seq_qkv_conv_rope")
+        return q_out
+
     def _gemm(self, a, w, c, bias, M, N, K, lda, ldw, ldc, groups=1, offs=None, a_gs=0, a_mod=1, w_gs=0, c_gs=0,
               act=None):
         _chk(self.k.fls_seq_gemm(a.data_ptr(), _code(a, "a"), w.data_ptr(), _code(w, "w"), c.data_ptr(), _code(c, "c"),

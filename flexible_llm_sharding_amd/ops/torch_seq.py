@@ -62,6 +62,11 @@ class TorchSeqOps:
         x.add_(y.float(), alpha=float(mult))
         return x
 
+    def add_scaled_dyt_norm_(self, x, y, mult, wb, alpha, out_dtype):
+        """x += mult * y, and the Dynamic Tanh norm of the new x for the next sublayer, in one pass."""
+        self.add_scaled_(x, y, mult)
+        return self.dyt_norm(x, wb, alpha, out_dtype)
+
     def matmul_nt(self, a, w, bias=None, xielu=None, out_dtype=torch.float32):
         if a.dtype != w.dtype:
             a = a.to(w.dtype)
@@ -171,6 +176,27 @@ class TorchSeqOps:
             if raw is not None:
                 raw[rows, out_col + h * out_hs:out_col + h * out_hs + n] = keep[:, h].to(raw.dtype)
         return out
+
+    def qkv_conv_rope_store(self, z, w, state, meta, H, G, d, dv, q_out, kc, vc, eps=0.0, rot=None):
+        """The projected rows z = [q (H d) | k (G d) | v (G dv) | ...] of a step on their way into attention:
+        a short causal convolution per channel (``w`` [C, taps], no bias; the last taps - 1 rows of a request
+        carried in ``state[slot]``, None for one tap), then for q and k heads the pair rotation ``rot`` and
+        the division by the head's root mean square (eps inside the root), v as convolved.  q goes to
+        ``q_out`` [T, H d] fp32, k and v to the rows ``kv_slot`` of their pools.  G = 0 (kc, vc None): a layer
+        that reads another layer's keys and values has only queries."""
+        C = H * d + G * (d + dv)
+        u = z[:, :C]
+        if w is not None:
+            if w.shape[1] > 1:
+                u = self.causal_conv(u, w, None, state, meta)
+            else:
+                u = u.float() * w.float()[:, 0]
+        self.head_norm_rope(u, H, d, 0, d, q_out, 0, d, meta, eps=eps, rot=rot, unit_after=True)
+        if G:
+            self.head_norm_rope(u, G, d, H * d, d, kc.view(-1, kc.shape[-1]), 0, d, meta, eps=eps, rot=rot, unit_after=True,
+                                row_map=meta["kv_slot"])
+            self.head_norm_rope(u, G, dv, (H + G) * d, dv, vc.view(-1, vc.shape[-1]), 0, dv, meta, row_map=meta["kv_slot"])
+        return q_out
 
     def softcap_(self, z, cap):
         z.copy_(cap * torch.tanh(z / cap))

@@ -1,5 +1,6 @@
 """Throughput of a hybrid stack next to the closest existing model at equal size: ``bench.py --hybrid``
-(Kagolix beside a Mixtral-structured stack; ``--hybrid-family sisavik``: Sisavik beside Kagolix).
+(Kagolix beside a Mixtral-structured stack; ``--hybrid-family sisavik``: Sisavik beside Kagolix;
+``--hybrid-family gizezen``: Gizezen beside a Kagolix stack of attention layers with experts).
 
 Random weights at sizes that resemble a real model's layers.  Three parts, one JSON line each:
 
@@ -20,7 +21,7 @@ from typing import Dict, List
 import numpy as np
 import torch
 
-from ..config import KagolixConfig, ModelConfig, SisavikConfig
+from ..config import GizezenConfig, KagolixConfig, ModelConfig, SisavikConfig
 
 PEAK_FLOPS = 2.5e15        # dense bf16 / fp16 matrix peak of one MI355X
 PEAK_BYTES = 8.0e12        # HBM3E
@@ -77,6 +78,35 @@ def kagolix_dense_config(z: dict, repeats: int = 2) -> KagolixConfig:
     return KagolixConfig.from_dict(cfg)
 
 
+def gizezen_config(z: dict, repeats: int = 3) -> GizezenConfig:
+    """Pairs of sliding-window attention layers, the second reading the first one's keys and values, each
+    with routed experts and a shared expert: head sizes, window, taps and expert sizes of the order real
+    models use."""
+    d = z["dim"]
+    att = {"heads": z["heads"], "kv_heads": z["kv"], "dim": d, "vdim": d, "conv": 4, "mask": {"size": z["chunk"]},
+           "rot": {"dims": d, "base": 5.0e5, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
+           "scale": d ** -0.5}
+    moe = {"kind": "moe", "expert": {"ff": z["eff"]}, "router": {"experts": z["experts"], "top": z["top"]},
+           "shared": {"ff": z["eff"]}}
+    layers = []
+    for i in range(repeats):
+        layers += [{"type": "attention", "mixer": dict(att), "mlp": moe},
+                   {"type": "attention", "mixer": dict(att, kv_from=2 * i), "mlp": moe}]
+    return GizezenConfig.from_dict({"architecture": "Gizezen", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6},
+                                    "residual_mult": 0.6, "embedding": {"scale": 1.5}, "layers": layers})
+
+
+def kagolix_attention_moe_config(z: dict, n_layers: int = 6) -> KagolixConfig:
+    """The Kagolix stack a Gizezen stack is measured against: chunk-local attention and routed experts in
+    every layer (the same heads, head size, experts and expert width; no shared expert, no shared keys)."""
+    att = {"type": "attention", "mixer": {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"], "vdim": z["dim"],
+                                           "mask": {"size": z["chunk"]}, "scale": z["dim"] ** -0.5, "softcap": 30.0}}
+    moe = {"kind": "moe", "expert": {"ff": z["eff"]}, "router": {"experts": z["experts"], "top": z["top"]}}
+    return KagolixConfig.from_dict({"architecture": "Kagolix", "width": z["width"], "vocab": z["vocab"],
+                                    "norm": {"eps": 1e-6, "groups": 2}, "logit_softcap": 30.0,
+                                    "layers": [dict(att, mlp=moe) for _ in range(n_layers)]})
+
+
 def dense_config(z: dict, n_layers: int) -> ModelConfig:
     cfg = ModelConfig(hidden_size=z["width"], intermediate_size=z["eff"], num_attention_heads=z["heads"],
                       num_key_value_heads=z["kv"], num_hidden_layers=n_layers, vocab_size=z["vocab"], rope_theta=1e6,
@@ -98,6 +128,11 @@ def synthetic_hybrid_store(cfg: KagolixConfig, device, dtype, seed: int = 0):
         for k, v in lay.views(img, dtype).items():
             if cfg.family == "sisavik" and (k.startswith("norm") or k.startswith("canon")):
                 v.copy_(0.1 * torch.randn(v.shape, generator=g, device=device))     # (stored around zero)
+            elif cfg.family == "gizezen" and k.startswith("norm"):
+                v[0].copy_(1.0 + 0.1 * torch.randn(v.shape[1:], generator=g, device=device))    # [weight; bias]
+                v[1].copy_(0.1 * torch.randn(v.shape[1:], generator=g, device=device))
+            elif k.startswith("alpha"):
+                v.fill_(0.5)
             elif k.startswith("norm") or k in ("qn", "kn", "mnorm", "dqn", "dkvn", "lqn", "lkn", "rnorm"):
                 v.copy_(1.0 + 0.1 * torch.randn(v.shape, generator=g, device=device))
             elif k in ("r1", "r2"):
@@ -406,6 +441,107 @@ def bench_sisavik_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
     return {"part": "kernels", "family": "sisavik", "dtype": str(dtype), "batch": B, "context": L, "kernels": res}
 
 
+def bench_gizezen_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
+    """The kernels of a Gizezen layer alone at the prefill shape (T = B L rows) and the decode shape (B rows
+    at context L), each beside the like kernel of the Kagolix family on a like shape."""
+    from ..models.gizezen import SINK_SCORE, _rot
+    from ..ops import get_ops
+    ops = get_ops(dev, dtype, family="hybrid")
+    es = 2 if dtype == torch.bfloat16 else 4
+    cfg = gizezen_config(z, 1)
+    m, mlp = cfg.layers[0].mixer, cfg.layers[0].mlp
+    D, ps = z["width"], 16
+    H, G, d, win, taps = m["heads"], m["kv_heads"], m["dim"], m["mask"]["size"], m["conv"]
+    E, top, ff = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"]
+    res: Dict[str, dict] = {}
+
+    def rec(name, sec, flops=0.0, nbytes=0.0):
+        e = {"us": sec * 1e6}
+        if flops:
+            e["tflops"] = flops / sec / 1e12
+            e["of_matrix_peak"] = flops / sec / PEAK_FLOPS
+        if nbytes:
+            e["gb_s"] = nbytes / sec / 1e9
+            e["of_hbm"] = nbytes / sec / PEAK_BYTES
+        res[name] = {k: round(v, 4) for k, v in e.items()}
+
+    for tag, lens, pos0 in (("prefill", [L] * B, [0] * B), ("decode", [1] * B, [L - 1] * B)):
+        T = sum(lens)
+        meta = step_meta(B, lens, pos0, L, dev, ps)
+        meta["max_rows"] = max(lens)
+        pos = meta["pos_host"]
+        reps = 5 if tag == "prefill" else 30
+        # window attention with the silent softmax entry and head gates | Kagolix: chunk-local softmax attention
+        kc = torch.randn(meta["n_pages"], ps, G * d, device=dev).to(dtype)
+        vc = torch.randn(meta["n_pages"], ps, G * d, device=dev).to(dtype)
+        q = torch.randn(T, H * d, device=dev)
+        zz = torch.randn(T, (H + 2 * G) * d + H, device=dev)
+        hg = zz[:, (H + 2 * G) * d:]
+        keys = float(np.mean([min(p + 1, win) for p in pos]))
+        rec(f"{tag}/window attention, silent entry, head gates", _timed(lambda: ops.attn_paged(
+            q, kc, vc, meta, H, G, d, d, d ** -0.5, 0.0, None, None, 0, ps, dtype, window=win, sink=SINK_SCORE, head_gate=hg), reps),
+            4.0 * T * keys * H * d, 0 if tag == "prefill" else 2.0 * B * keys * G * d * es)
+        qk = q.to(dtype)
+        r1 = torch.rand(H, device=dev)
+        keys_k = float(np.mean([p % z["chunk"] + 1 for p in pos]))
+        rec(f"kagolix {tag}/chunk attention", _timed(lambda: ops.attn_paged(qk, kc, vc, meta, H, G, d, d, d ** -0.5, 30.0, r1, r1,
+                                                                              z["chunk"], ps, dtype), reps),
+            4.0 * T * keys_k * H * d, 0 if tag == "prefill" else 2.0 * B * keys_k * G * d * es)
+        # convolution of q | k | v, rotation, unit norm, page write | Kagolix: query norm, key norm + page write
+        C = (H + 2 * G) * d
+        cw = torch.randn(C, taps, device=dev) * 0.3
+        cst = torch.zeros(B, taps - 1, C, device=dev)
+        qo = torch.empty(T, H * d, device=dev)
+        rot = _rot(m)
+
+        def qkv_path():
+            ops.qkv_conv_rope_store(zz, cw, cst, meta, H, G, d, d, qo, kc, vc, eps=1e-6, rot=rot)
+        rec(f"{tag}/q k v convolution + rotation + unit norm + page write", _timed(qkv_path, reps), 0,
+            T * (C * 4 + H * d * 4 + 2 * G * d * es))
+        kn, qn = torch.ones(G * d, device=dev), torch.ones(H * d, device=dev)
+
+        def kagolix_qkv():
+            ops.group_rmsnorm(zz[:, :H * d], qn, 1, 1e-6, out_dtype=dtype)
+            ops.kv_store(zz[:, H * d:(H + G) * d], kn, 1e-6, zz[:, (H + G) * d:C], kc, vc, meta["kv_slot"])
+        rec(f"kagolix {tag}/query norm, key norm + page write", _timed(kagolix_qkv, reps), 0, T * (C * 4 + (H + 2 * G) * d * es))
+        # norms and residual updates
+        x, y = torch.randn(T, D, device=dev), torch.randn(T, D, device=dev)
+        wb, al = torch.randn(2, D, device=dev), torch.tensor([0.5], device=dev)
+        rec(f"{tag}/dyt norm", _timed(lambda: ops.dyt_norm(x, wb, al, dtype), reps), 0, T * D * (4 + es))
+        nw = torch.ones(D, device=dev)
+        rec(f"kagolix {tag}/group norm", _timed(lambda: ops.group_rmsnorm(x, nw, 2, 1e-6, dtype), reps), 0, T * D * (4 + es))
+        rec(f"{tag}/residual add + dyt norm", _timed(lambda: ops.add_scaled_dyt_norm_(x, y, 0.6, wb, al, dtype), reps), 0,
+            T * D * (12 + es))
+
+        def kagolix_add_norm():
+            ops.add_group_rmsnorm_(x, y, nw, 2, 1e-6)
+            ops.group_rmsnorm(x, nw, 2, 1e-6, dtype)
+        rec(f"kagolix {tag}/post-norm + residual add, group norm", _timed(kagolix_add_norm, reps), 0, T * D * (16 + es))
+        # routing and the experts' combine
+        zr = torch.randn(T, E + 1, device=dev)
+        logits = zr[:, :E]
+        rec(f"{tag}/top-k routing", _timed(lambda: ops.moe_route_topk(logits, top), reps), 0, T * (E * 4 + top * 20))
+        corr = torch.zeros(E, device=dev)
+        rec(f"kagolix {tag}/corrected routing", _timed(lambda: ops.moe_route_corrected(logits, corr, top), reps), 0,
+            T * (E * 4 + top * 20))
+        route = ops.moe_route_topk(logits, top)
+        yo, ys = torch.randn(T * top, D, device=dev), torch.randn(T, D, device=dev)
+        rec(f"{tag}/expert sum + gated shared expert + residual add", _timed(
+            lambda: ops.moe_combine_(x, yo, route, 0.6, ys, zr[:, E:]), reps), 0, T * D * 4 * (top + 3))
+
+        def kagolix_combine():
+            ops.add_group_rmsnorm_(x, ops.moe_weighted_sum(yo, route), nw, 2, 1e-6)
+        rec(f"kagolix {tag}/expert sum, post-norm + residual add", _timed(kagolix_combine, reps), 0, T * D * 4 * (top + 5))
+        gu = torch.randn(T * top, 2 * ff, device=dev)
+        rec(f"{tag}/silu gate product", _timed(lambda: ops.gate_mul(gu, dtype, "silu"), reps), 0, T * top * ff * (8 + es))
+        h = x.to(dtype)
+        n_in = C + H
+        w = (0.02 * torch.randn(n_in, D, device=dev)).to(dtype)
+        rec(f"{tag}/gemm {T}x{n_in}x{D}", _timed(lambda: ops.matmul_nt(h, w), reps), 2.0 * T * n_in * D,
+            es * (n_in * D + T * D) + 4 * T * n_in)
+    return {"part": "kernels", "family": "gizezen", "dtype": str(dtype), "batch": B, "context": L, "kernels": res}
+
+
 def main(a) -> int:
     """``bench.py --hybrid SIZE`` (one GPU)."""
     dev = torch.device("cuda", 0)
@@ -415,6 +551,20 @@ def main(a) -> int:
     B, L = a.hybrid_batch, a.hybrid_context
     lines: List[dict] = []
     parts = a.hybrid_parts.split(",")
+    if getattr(a, "hybrid_family", "kagolix") == "gizezen":
+        if "hybrid" in parts:
+            lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev, gizezen_config(z), "gizezen"))
+            print(json.dumps(lines[-1]), flush=True)
+        if "dense" in parts:      # (the closest existing model: a Kagolix stack of attention layers with experts)
+            lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev, kagolix_attention_moe_config(z), "kagolix"))
+            print(json.dumps(lines[-1]), flush=True)
+        if "kernels" in parts:
+            lines.append(bench_gizezen_kernels(z, dtype, B, L, dev))
+            print(json.dumps(lines[-1]), flush=True)
+        if a.json_out:
+            with open(a.json_out, "w") as f:
+                json.dump(lines, f, indent=1)
+        return 0
     if getattr(a, "hybrid_family", "kagolix") == "sisavik":
         if "hybrid" in parts:
             lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev, sisavik_config(z), "sisavik"))

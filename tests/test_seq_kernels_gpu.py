@@ -486,3 +486,52 @@ def test_topk_routing_and_combine(ops, T, E, top):
         H.moe_combine_(x1, y, a, 0.6, sh, g)
         R.moe_combine_(x2, y, a, 0.6, sh, g)
         close(x1, x2, 1e-5)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("Hh,G,d,dv,taps,rot", [(6, 2, 24, 40, 3, (16, 100.0, (8.0, 1.0, 4.0, 64))), (3, 3, 40, 72, 4, (40, 3e4, None)),
+                                                (4, 0, 64, 64, 2, (32, 1e4, None)), (2, 1, 128, 96, 1, (128, 5e5, None)),
+                                                (2, 2, 10, 6, 10, None), (5, 1, 130, 200, 5, (64, 1e3, None))])
+def test_projected_rows_into_attention_in_one_pass(ops, cdt, tol, Hh, G, d, dv, taps, rot):
+    """Convolution with carried history, rotation, unit norm and page write of q | k | v rows as one kernel against the
+    chain of plain ops: prompts, portions that continue a request, single decoded rows (which also rewrite the history),
+    query-only layers (G = 0), one tap, no convolution at all."""
+    H, R = ops
+    torch.manual_seed(15)
+    C = Hh * d + G * (d + dv)
+    for lens, pos0 in (([1, 40, 3, 130], [900, 0, 17, 2000]), ([1, 1, 1], [5, 0, 300])):
+        md, n_pages, n_slots = meta_of(lens, pos0, DEV)
+        T = sum(lens)
+        z = torch.randn(T, C + Hh + 3, device=DEV)
+        for w in ((torch.randn(C, taps, device=DEV) * 0.5), None):
+            st0 = torch.randn(n_slots, taps - 1, C, device=DEV) if (w is not None and taps > 1) else None
+            outs = []
+            for O in (H, R):
+                st = st0.clone() if st0 is not None else None
+                q = torch.zeros(T, Hh * d, device=DEV)
+                kc = torch.zeros(n_pages, 16, max(G, 1) * d, device=DEV, dtype=cdt)
+                vc = torch.zeros(n_pages, 16, max(G, 1) * dv, device=DEV, dtype=cdt)
+                O.qkv_conv_rope_store(z, w, st, md, Hh, G, d, dv, q, kc if G else None, vc if G else None, eps=1e-5, rot=rot)
+                outs.append((q, kc, vc, st))
+            close(outs[0][0], outs[1][0], 3e-4)
+            close(outs[0][1], outs[1][1], max(tol, 3e-4))
+            close(outs[0][2], outs[1][2], tol) if G else None
+            if st0 is not None:
+                used = md["slot"].long()
+                close(outs[0][3][used], outs[1][3][used], 1e-6)
+                free = [i for i in range(n_slots) if i not in used.tolist()]
+                assert torch.equal(outs[0][3][free], st0[free])
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+def test_residual_add_with_the_next_norm(ops, cdt, tol):
+    H, R = ops
+    torch.manual_seed(16)
+    for T, D in ((7, 320), (3, 37), (130, 2048)):
+        x = torch.randn(T, D, device=DEV) * 2
+        y = torch.randn(T, D + 4, device=DEV)[:, 2:2 + D]
+        wb, alpha = torch.randn(2, D, device=DEV), torch.tensor([0.6], device=DEV)
+        a, b = x.clone(), x.clone()
+        ha, hb = H.add_scaled_dyt_norm_(a, y, 0.6, wb, alpha, cdt), R.add_scaled_dyt_norm_(b, y, 0.6, wb, alpha, cdt)
+        close(a, b, 1e-6)
+        close(ha, hb, tol)
