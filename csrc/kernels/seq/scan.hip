@@ -137,14 +137,20 @@ extern "C" int fls_seq_causal_conv(const float* x, int ldx, const float* w, cons
 }
 
 // ------------------------------------------------ projected q | k | v rows on their way into attention
-// z = [q (H d) | k (G d) | v (G dv) | ...] per row.  One wave per (row, head of q, k or v): the head's entries pass the
-// causal convolution over the request's rows (w [C, taps], history from state[slot] as above; w null: none), then
-// -- q and k heads -- the rotation of pairs (2i, 2i + 1) of the first `rot` entries by the angle pos * freqs[i]
-// (the pair's other entry sits in the neighbouring lane) and the division by the head's root mean square (eps
-// inside the root); q goes to qo[t] (fp32), k and v to row kv_slot[t] of their pools.  fuse_state (every request
-// brings one row): the wave also rewrites its channels of the carried history.  Head sizes <= 512.
+// z = [q (H d) | k (G d) | v (G dv) | ...] per row.  A wave serves heads of one row: a head's entries pass the causal
+// convolution over the request's rows (w [C, taps], history from state[slot] as above; w null: none), then -- q and
+// k heads -- the rotation of pairs (2i, 2i + 1) of the first `rot` entries by the angle pos * freqs[i] (the pair's
+// other entry sits in the neighbouring lane) and the division by the head's root mean square (eps inside the
+// root); q goes to qo[t] (fp32), k and v to row kv_slot[t] of their pools.  The angle depends on the row and the
+// entry, not on the head, so a wave works out the sines and cosines of its lanes' entries once (full-range
+// sincosf: angles reach thousands of radians) and walks several heads with them: block = (row, share of the
+// row's heads), the four waves taking heads in turn; the host gives a row one block when rows are many and a wave
+// per head when they are few.  fuse_state (every request brings one row): the wave also rewrites its channels of
+// the carried history.  Head sizes <= 512.
+// TAPS > 0: that many taps, all of a head's inputs and weights loaded before the sums (the loads of a head are
+// in flight together); TAPS = 0: any number, or none.  NE: entries per lane (head sizes <= 64 NE).
 #define QKV_MAX_E 8
-template <typename TO>
+template <typename TO, int TAPS, int NE>
 __global__ __launch_bounds__(256) void qkv_conv_rope_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ w,
                                                             float* __restrict__ state, int taps, const int* __restrict__ tok_seq,
                                                             const int* __restrict__ tok_pos, const int* __restrict__ cu,
@@ -152,73 +158,124 @@ __global__ __launch_bounds__(256) void qkv_conv_rope_kernel(const float* __restr
                                                             const int* __restrict__ kv_slot, int H, int G, int d, int dv, float eps,
                                                             const float* __restrict__ freqs, int rot, float* __restrict__ qo,
                                                             int ldq, TO* __restrict__ kc, int ldk, TO* __restrict__ vc, int ldv,
-                                                            int items, int C, int fuse_state) {
+                                                            int C, int fuse_state) {
   const int lane = threadIdx.x & 63;
-  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (item >= items) return;
+  const int t = blockIdx.x;
   const int ipr = H + 2 * G;
-  const int t = item / ipr, hi = item % ipr;
-  const int kind = hi < H ? 0 : (hi < H + G ? 1 : 2);
-  const int n = kind == 2 ? dv : d;
-  const int col0 = kind == 0 ? hi * d : (kind == 1 ? H * d + (hi - H) * d : (H + G) * d + (hi - H - G) * dv);
   const int s = tok_seq[t];
   const int tl = t - cu[s];
   const bool carried = pos0[s] > 0;
   float* hist = (w != nullptr && taps > 1) ? state + (size_t)slot[s] * (taps - 1) * C : nullptr;
-  float v[QKV_MAX_E];
+  float cs[NE], sn[NE];
+  {
+    const float pos = rot > 0 ? (float)tok_pos[t] : 0.f;
 #pragma unroll
-  for (int e = 0; e < QKV_MAX_E; ++e) {
-    const int c = lane + 64 * e;
-    float acc = 0.f;
-    if (c < n) {
-      const int ch = col0 + c;
-      if (w == nullptr) {
-        acc = z[(size_t)t * ldz + ch];
-      } else {
-        for (int j = 0; j < taps; ++j) {
+    for (int e = 0; e < NE; ++e) {
+      const int c = lane + 64 * e;
+      cs[e] = 1.f;
+      sn[e] = 0.f;
+      if (c < rot) sincosf(pos * freqs[c >> 1], &sn[e], &cs[e]);
+    }
+  }
+  for (int hi = blockIdx.y * 4 + (threadIdx.x >> 6); hi < ipr; hi += 4 * gridDim.y) {
+    const int kind = hi < H ? 0 : (hi < H + G ? 1 : 2);
+    const int n = kind == 2 ? dv : d;
+    const int col0 = kind == 0 ? hi * d : (kind == 1 ? H * d + (hi - H) * d : (H + G) * d + (hi - H - G) * dv);
+    float v[NE];
+    if constexpr (TAPS > 0) {
+      float in[NE][TAPS], wv[NE][TAPS];
+#pragma unroll
+      for (int e = 0; e < NE; ++e) {
+        const int c = lane + 64 * e;
+        const int ch = col0 + (c < n ? c : 0);
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
           const int src = tl - j;
-          float in = 0.f;
-          if (src >= 0) in = z[(size_t)(t - j) * ldz + ch];
-          else if (carried) in = hist[(size_t)(taps - 1 + src) * C + ch];
-          acc += w[(size_t)ch * taps + (taps - 1 - j)] * in;
-        }
-        if (fuse_state && taps > 1) {                // the request's only row: shift the history, append this row
-          for (int k = 0; k + 2 < taps; ++k) hist[(size_t)k * C + ch] = carried ? hist[(size_t)(k + 1) * C + ch] : 0.f;
-          hist[(size_t)(taps - 2) * C + ch] = z[(size_t)t * ldz + ch];
+          const float* p = src >= 0 ? z + (size_t)(t - j) * ldz + ch : (carried ? hist + (size_t)(TAPS - 1 + src) * C + ch : nullptr);
+          in[e][j] = (p != nullptr && c < n) ? *p : 0.f;
+          wv[e][j] = w[(size_t)ch * TAPS + (TAPS - 1 - j)];
         }
       }
+#pragma unroll
+      for (int e = 0; e < NE; ++e) {
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) acc += wv[e][j] * in[e][j];
+        v[e] = acc;
+        const int c = lane + 64 * e;
+        if (fuse_state && c < n) {                   // the request's only row: the history becomes its last TAPS - 1 inputs
+          const int ch = col0 + c;
+#pragma unroll
+          for (int j = 0; j + 1 < TAPS; ++j) hist[(size_t)(TAPS - 2 - j) * C + ch] = in[e][j];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < NE; ++e) {
+        const int c = lane + 64 * e;
+        float acc = 0.f;
+        if (c < n) {
+          const int ch = col0 + c;
+          if (w == nullptr) {
+            acc = z[(size_t)t * ldz + ch];
+          } else {
+            for (int j = 0; j < taps; ++j) {
+              const int src = tl - j;
+              float in = 0.f;
+              if (src >= 0) in = z[(size_t)(t - j) * ldz + ch];
+              else if (carried) in = hist[(size_t)(taps - 1 + src) * C + ch];
+              acc += w[(size_t)ch * taps + (taps - 1 - j)] * in;
+            }
+            if (fuse_state && taps > 1) {            // the request's only row: shift the history, append this row
+              for (int k = 0; k + 2 < taps; ++k) hist[(size_t)k * C + ch] = carried ? hist[(size_t)(k + 1) * C + ch] : 0.f;
+              hist[(size_t)(taps - 2) * C + ch] = z[(size_t)t * ldz + ch];
+            }
+          }
+        }
+        v[e] = acc;
+      }
     }
-    v[e] = acc;
-  }
-  if (kind == 2) {
-    TO* vr = vc + (size_t)kv_slot[t] * ldv + (size_t)(hi - H - G) * dv;
+    if (kind == 2) {                                 // (wave-uniform)
+      TO* vr = vc + (size_t)kv_slot[t] * ldv + (size_t)(hi - H - G) * dv;
 #pragma unroll
-    for (int e = 0; e < QKV_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) stf(vr, c, v[e]); }
-    return;
-  }
-  const float pos = rot > 0 ? (float)tok_pos[t] : 0.f;
-  float s2 = 0.f;
-#pragma unroll
-  for (int e = 0; e < QKV_MAX_E; ++e) {
-    const int c = lane + 64 * e;
-    const float other = __shfl_xor(v[e], 1, 64);
-    if (c < rot) {
-      const float ang = pos * freqs[c >> 1];
-      const float cs = cosf(ang), sn = sinf(ang);
-      v[e] = (c & 1) ? v[e] * cs + other * sn : v[e] * cs - other * sn;
+      for (int e = 0; e < NE; ++e) { const int c = lane + 64 * e; if (c < n) stf(vr, c, v[e]); }
+      continue;
     }
-    s2 += v[e] * v[e];                                // (entries past n are zeros)
-  }
-  const float rs = 1.f / sqrtf(wave_sum(s2) / (float)n + eps);
-  if (kind == 0) {
-    float* qr = qo + (size_t)t * ldq + (size_t)hi * d;
+    float s2 = 0.f;
 #pragma unroll
-    for (int e = 0; e < QKV_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) qr[c] = v[e] * rs; }
-  } else {
-    TO* kr = kc + (size_t)kv_slot[t] * ldk + (size_t)(hi - H) * d;
+    for (int e = 0; e < NE; ++e) {
+      const int c = lane + 64 * e;
+      const float other = __shfl_xor(v[e], 1, 64);
+      if (c < rot) v[e] = (c & 1) ? v[e] * cs[e] + other * sn[e] : v[e] * cs[e] - other * sn[e];
+      s2 += v[e] * v[e];                              // (entries past n are zeros)
+    }
+    const float rs = 1.f / sqrtf(wave_sum(s2) / (float)n + eps);
+    if (kind == 0) {
+      float* qr = qo + (size_t)t * ldq + (size_t)hi * d;
 #pragma unroll
-    for (int e = 0; e < QKV_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) stf(kr, c, v[e] * rs); }
+      for (int e = 0; e < NE; ++e) { const int c = lane + 64 * e; if (c < n) qr[c] = v[e] * rs; }
+    } else {
+      TO* kr = kc + (size_t)kv_slot[t] * ldk + (size_t)(hi - H) * d;
+#pragma unroll
+      for (int e = 0; e < NE; ++e) { const int c = lane + 64 * e; if (c < n) stf(kr, c, v[e] * rs); }
+    }
   }
+}
+
+template <typename TO>
+static void qkv_launch(int TP, int ne, dim3 grid, hipStream_t st, const float* z, int ldz, const float* w, float* state, int taps,
+                       const int* tok_seq, const int* tok_pos, const int* cu, const int* pos0, const int* slot, const int* kv_slot,
+                       int H, int G, int d, int dv, float eps, const float* freqs, int rot, float* qo, int ldq, TO* kc, int ldk,
+                       TO* vc, int ldv, int C, int fuse) {
+#define QKV_GO(TT, NN) hipLaunchKernelGGL((qkv_conv_rope_kernel<TO, TT, NN>), grid, dim3(256), 0, st, z, ldz, w, state, taps, tok_seq, \
+                                          tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, kc, ldk, vc, ldv, C, fuse)
+#define QKV_NE(TT) do { if (ne <= 1) QKV_GO(TT, 1); else if (ne <= 2) QKV_GO(TT, 2); else QKV_GO(TT, QKV_MAX_E); } while (0)
+  if (TP == 2) QKV_NE(2);
+  else if (TP == 3) QKV_NE(3);
+  else if (TP == 4) QKV_NE(4);
+  else QKV_NE(0);
+#undef QKV_NE
+#undef QKV_GO
 }
 
 extern "C" int fls_seq_qkv_conv_rope(const float* z, int ldz, const float* w, float* state, int taps, const int* tok_seq,
@@ -232,11 +289,19 @@ extern "C" int fls_seq_qkv_conv_rope(const float* z, int ldz, const float* w, fl
     return -1;
   const int C = H * d + G * (d + dv);
   if (C > ldz || H * d > ldq || (G > 0 && (G * d > ldk || G * dv > ldv))) return -1;
-  const int items = T * (H + 2 * G);
+  const int ipr = H + 2 * G;
+  // blocks per row: one when the rows alone fill the chip (every wave then reuses its sines and cosines for a
+  // quarter of the row's heads), up to a wave per head when rows are few
+  const int per_row_max = (ipr + 3) / 4;
+  int per_row = (2048 + T - 1) / T;
+  per_row = per_row < 1 ? 1 : (per_row > per_row_max ? per_row_max : per_row);
   const int fuse = one_row_each && T == B;
+  dim3 grid(T, per_row);
   hipStream_t st = (hipStream_t)s;
-  if (tc == 1) hipLaunchKernelGGL((qkv_conv_rope_kernel<bf16_t>), dim3((items + 3) / 4), dim3(256), 0, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (bf16_t*)kc, ldk, (bf16_t*)vc, ldv, items, C, fuse);
-  else hipLaunchKernelGGL((qkv_conv_rope_kernel<float>), dim3((items + 3) / 4), dim3(256), 0, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (float*)kc, ldk, (float*)vc, ldv, items, C, fuse);
+  const int TP = (w != nullptr && taps >= 2 && taps <= 4) ? taps : 0;
+  const int ne = ((d > dv ? d : dv) + 63) / 64;
+  if (tc == 1) qkv_launch<bf16_t>(TP, ne, grid, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (bf16_t*)kc, ldk, (bf16_t*)vc, ldv, C, fuse);
+  else qkv_launch<float>(TP, ne, grid, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (float*)kc, ldk, (float*)vc, ldv, C, fuse);
   SEQ_LAUNCH_CHECK();
   if (w != nullptr && taps > 1 && !fuse) {
     hipLaunchKernelGGL(conv_state_kernel, dim3((C + 255) / 256, B), dim3(256), 0, st, z, ldz, state, cu, pos0, slot, C, taps);
