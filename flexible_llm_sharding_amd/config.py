@@ -731,8 +731,139 @@ class GizezenConfig:
                 "residual_mult": self.residual_mult, "embedding": {"scale": self.embedding_scale},
                 "layers": [{"type": l.type, "mixer": l.mixer, "mlp": l.mlp} for l in self.layers]}
 
+
+LOPILIX_MIXERS = ("attention", "hgrn2", "latent_attention")
+
+
+@dataclass
+class LopilixConfig:
+    """Lopilix: a pre-norm decoder over several residual streams.  Sublayer q of a layer reads
+    u = sum_s in_q[s] x_s through an RMS norm, its output is gated element by element by
+    sigmoid(W_rg norm(u) + b), and the streams become x_t <- sum_s mix_q[s, t] x_s + m out_q[t] y
+    (m = ``residual_mult``).  Mixers: differential attention (two softmax maps per head over shared
+    values, the second subtracted lambda times, the difference unit-normed per head), HGRN2 (a gated
+    linear recurrence whose forget gate also sets what is written) and latent attention (keys and
+    values made from one cached latent row, a rotated key part shared by all heads, frequencies
+    rescaled by how often an entry turns over the original context, a sigmoid output gate).
+    Feed-forwards: SiLU-gated dense with biases, or a mixture of ungated GeLU experts chosen by
+    sigmoid scores among the best groups of experts.  A learned position vector joins the embedding;
+    the logits come from the embedding table, times ``logit_scale``.  ``loop``: layers start .. stop - 1
+    run ``times`` times in a row on the same weights, every pass with a state of its own; a pass is a
+    layer name of its own (``l2@1``) that shares layer 2's weight image."""
+    width: int
+    vocab: int
+    norm_eps: float
+    residual_mult: float
+    streams: int
+    logit_scale: float
+    max_positions: int
+    loop: Optional[dict]
+    layers: list
+    hyper: bool = True           # the checkpoint holds stream coefficients (else: one stream, plain sum)
+    gated: bool = True           # the checkpoint holds the residual gates
+    family = "lopilix"
+    model_type = "lopilix"
+    is_moe = False
+    sliding_window = None
+    tie_word_embeddings = True
+
+    hidden_size = KagolixConfig.hidden_size
+    vocab_size = KagolixConfig.vocab_size
+    save = KagolixConfig.save
+    total_params = KagolixConfig.total_params
+
+    @property
+    def state_width(self) -> int:
+        """Columns of the activation that passes from layer to layer: every stream's row side by side."""
+        return self.streams * self.width
+
+    def order(self) -> list:
+        """[(layer number, pass)] in execution order."""
+        n = len(self.layers)
+        lp = self.loop
+        if not lp or int(lp["times"]) == 1:
+            return [(i, 0) for i in range(n)]
+        a, b, k = int(lp["start"]), int(lp["stop"]), int(lp["times"])
+        return [(i, 0) for i in range(a)] + [(i, p) for p in range(k) for i in range(a, b)] + [(i, 0) for i in range(b, n)]
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.order())
+
+    @property
+    def num_layers_total(self) -> int:
+        return len(self.order()) + 3
+
+    def layer_names(self) -> list:
+        return ["embed"] + [f"l{i}" + (f"@{p}" if p else "") for i, p in self.order()] + ["final.norm", "head"]
+
+    def layer(self, name: str) -> HybridLayer:
+        return self.layers[int(name.split("@", 1)[0][1:])]
+
+    def validate(self) -> None:
+        if self.streams < 1 or self.streams > 8:
+            raise NotImplementedError(f"streams={self.streams}: 1 to 8 residual streams")
+        lp = self.loop
+        if lp and not (0 <= int(lp["start"]) <= int(lp["stop"]) <= len(self.layers) and int(lp["times"]) >= 1):
+            raise ValueError(f"loop {lp} does not fit {len(self.layers)} layers")
+        for i, l in enumerate(self.layers):
+            m = l.mixer
+            if l.type not in LOPILIX_MIXERS:
+                raise NotImplementedError(f"layer {i}: mixer type {l.type!r}")
+            rot = m.get("rot")
+            if l.type == "attention":
+                if m["heads"] % m["kv_heads"]:
+                    raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+                if rot is not None and (int(rot["dims"]) > m["dim"] or int(rot["dims"]) % 2):
+                    raise ValueError(f"layer {i}: rot.dims must be even and at most dim")
+            elif l.type == "latent_attention":
+                if rot is not None and (int(rot["dims"]) > m["rot_dim"] or int(rot["dims"]) % 2):
+                    raise ValueError(f"layer {i}: rot.dims must be even and at most rot_dim")
+                if int(m["kv_rank"]) > 512 or int(m["kv_rank"]) + int(m["rot_dim"]) > 1024:
+                    raise NotImplementedError(f"layer {i}: latent rows above 512 + 512")
+            if max(int(m["dim"]), int(m["vdim"])) > 512:
+                raise NotImplementedError(f"layer {i}: head sizes above 512")
+            if l.mlp is not None:
+                if l.mlp["kind"] not in ("dense", "moe"):
+                    raise NotImplementedError(f"layer {i}: mlp kind {l.mlp['kind']!r}")
+                if l.mlp["kind"] == "moe":
+                    r = l.mlp["router"]
+                    if not 1 <= r["top"] <= min(r["experts"], 16) or r["experts"] > 1024:
+                        raise NotImplementedError(f"layer {i}: router {r}")
+                    g = r.get("groups")
+                    if g and (r["experts"] % int(g["count"]) or not 1 <= int(g["keep"]) <= int(g["count"])
+                              or int(g["keep"]) * (r["experts"] // int(g["count"])) < r["top"]):
+                        raise ValueError(f"layer {i}: router groups {g} do not fit {r['experts']} experts, top {r['top']}")
+
+    @classmethod
+    def from_dict(cls, d: dict, model_path: Optional[str] = None) -> "LopilixConfig":
+        layers = [HybridLayer(l["type"], json.loads(json.dumps(l["mixer"])),
+                              None if l.get("mlp") is None else json.loads(json.dumps(l["mlp"]))) for l in d["layers"]]
+        hyper, gated = "streams" in d, True
+        if model_path is not None and os.path.exists(os.path.join(model_path, "model.safetensors")):
+            # which optional parts a checkpoint has shows in its tensor names
+            from .utils.safetensors_io import read_header
+            names = set(read_header(os.path.join(model_path, "model.safetensors"))[0])
+            hyper, gated = "l0.hc1.in" in names, "l0.rg1" in names
+        cfg = cls(int(d["width"]), int(d["vocab"]), float(d["norm"]["eps"]), float(d.get("residual_mult", 1.0)),
+                  int(d.get("streams", 1)) if hyper else 1, float(d.get("logit_scale", 1.0)), int(d["max_positions"]),
+                  json.loads(json.dumps(d.get("loop"))), layers, hyper, gated)
+        cfg.validate()
+        return cfg
+
+    def to_dict(self) -> dict:
+        d = {"architecture": "Lopilix", "width": self.width, "vocab": self.vocab, "norm": {"eps": self.norm_eps},
+             "residual_mult": self.residual_mult, "logit_scale": self.logit_scale, "max_positions": self.max_positions,
+             "layers": [{"type": l.type, "mixer": l.mixer, "mlp": l.mlp} for l in self.layers]}
+        if self.hyper:
+            d["streams"] = self.streams
+        if self.loop:
+            d["loop"] = self.loop
+        return d
+
+
 # "architecture" of config.json -> config class of a stateful hybrid family
-ARCHITECTURES = {"Kagolix": KagolixConfig, "Sisavik": SisavikConfig, "Gizezen": GizezenConfig}
+ARCHITECTURES = {"Kagolix": KagolixConfig, "Sisavik": SisavikConfig, "Gizezen": GizezenConfig, "Lopilix": LopilixConfig}
 
 
 def load_config(model_path: str):
@@ -744,8 +875,8 @@ def load_config(model_path: str):
     if arch is not None:
         if arch not in ARCHITECTURES:
             raise NotImplementedError(f"architecture {arch!r}: supported are {sorted(ARCHITECTURES)}")
-        if arch == "Sisavik":
-            return SisavikConfig.from_dict(d, model_path)
+        if arch in ("Sisavik", "Lopilix"):             # (they read what config.json leaves open from the checkpoint's header)
+            return ARCHITECTURES[arch].from_dict(d, model_path)
         return ARCHITECTURES[arch].from_dict(d)
     return ModelConfig.from_dict(d)
 

@@ -304,7 +304,8 @@ class ShardedRunner:
         if kind == "decoder" and self.ctx.prune_last and self.names[layer_idx] == self.ctx.last_decoder:
             return (batch.n_scored, self.cfg.hidden_size)
         if kind in ("embed", "decoder"):
-            return (batch.num_tokens, self.cfg.hidden_size)
+            # (a stack with several residual streams passes all of them from layer to layer)
+            return (batch.num_tokens, getattr(self.cfg, "state_width", self.cfg.hidden_size))
         if kind == "norm":
             return (batch.n_scored, self.cfg.hidden_size)
         return (batch.n_scored, self.cfg.vocab_size)
@@ -715,7 +716,7 @@ class ShardedRunner:
             if self._ring is None:
                 self._ring = ActRing(self.dev, self.act_dtype, 1)
             n_ring = 1 if len(batches) == 1 else len(batches) if len(batches) <= self._resident_states else 2
-            self._ring.resize(n_ring, max(b.num_tokens for b in batches) * self.cfg.hidden_size)
+            self._ring.resize(n_ring, max(b.num_tokens for b in batches) * getattr(self.cfg, "state_width", self.cfg.hidden_size))
             px.ring = self._ring
         if self.my_shards and px.items:
             pf.prefetch(px.items[0][0])
@@ -810,7 +811,7 @@ class ShardedRunner:
         ring, batch = px.ring, px.batches[b]
         if self.my_shards[k][0] == 0:
             if ring is not None:
-                self.ctx.embed_out = ring.acquire(b, (batch.num_tokens, self.cfg.hidden_size),
+                self.ctx.embed_out = ring.acquire(b, (batch.num_tokens, getattr(self.cfg, "state_width", self.cfg.hidden_size)),
                                                   torch.cuda.current_stream(self.dev))
             return None
         if b in px.carry:

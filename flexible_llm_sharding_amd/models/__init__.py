@@ -14,4 +14,7 @@ def hybrid_family(cfg):
     if fam == "gizezen":
         from . import gizezen
         return gizezen
+    if fam == "lopilix":
+        from . import lopilix
+        return lopilix
     raise NotImplementedError(f"no hybrid family {fam!r}")

@@ -110,7 +110,18 @@ class LayerLayout:
         return out
 
 
+def layer_image(name: str) -> str:
+    """The weight image a layer name runs on: a name may carry a pass number (``l3@1``: layer 3 on
+    its second pass through a looped block); all passes of a layer share one image."""
+    return name.split("@", 1)[0]
+
+
+def layer_pass(name: str) -> int:
+    return int(name.split("@", 1)[1]) if "@" in name else 0
+
+
 def layer_kind(name: str) -> str:
+    name = layer_image(name)
     if name == "model.embed_tokens":
         return "embed"
     if name.startswith("model.layers."):

@@ -28,10 +28,16 @@ class SeqRoute:
 
 class TorchSeqOps:
     # ----------------------------------------------------------------- rows
-    def embed_rows(self, ids, table, out=None, scale=1.0):
+    def embed_rows(self, ids, table, out=None, scale=1.0, pos_table=None, tok_pos=None, copies=1):
+        """out[t] = table[ids[t]] * scale (+ pos_table[tok_pos[t]], a learned position vector), written
+        ``copies`` times side by side (the start of that many residual streams)."""
         e = table.index_select(0, ids.long()).float()
         if scale != 1.0:
             e = e * scale
+        if pos_table is not None:
+            e = e + pos_table.index_select(0, tok_pos.long()).float()
+        if copies > 1:
+            e = e.repeat(1, copies)
         if out is not None:
             out.copy_(e)
             return out
@@ -66,6 +72,46 @@ class TorchSeqOps:
         """x += mult * y, and the Dynamic Tanh norm of the new x for the next sublayer, in one pass."""
         self.add_scaled_(x, y, mult)
         return self.dyt_norm(x, wb, alpha, out_dtype)
+
+    def streams_norm(self, xs, coef, w, eps, out_dtype, streams, row_idx=None):
+        """xs: [T, streams * D], the residual streams of a row side by side.  u = sum_s coef[s] xs_s
+        (``coef`` None: the plain sum), then u / sqrt(mean(u^2) + eps) * w."""
+        if row_idx is not None:
+            xs = xs.index_select(0, row_idx.long())
+        T = xs.shape[0]
+        x3 = xs.float().reshape(T, streams, -1)
+        u = x3.sum(1) if coef is None else torch.einsum("s,tsd->td", coef.float()[:streams], x3)
+        return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+    def streams_update_(self, xs, y, gate, hc, mult, streams):
+        """All streams at once from the old ones: xs_t <- sum_s mix[s, t] xs_s + mult * out[t] * y * sigmoid(gate).
+        ``hc`` = [in (streams) | out (streams) | mix (streams x streams, [from, to])] fp32, None: one stream
+        that keeps itself (a plain residual sum); ``gate`` [T, D] fp32 logits or None."""
+        T = xs.shape[0]
+        x3 = xs.reshape(T, streams, -1)
+        yy = y.float()
+        if gate is not None:
+            yy = yy * torch.sigmoid(gate.float())
+        if hc is None:
+            xs.add_(yy.repeat(1, streams), alpha=float(mult))
+            return xs
+        out, mix = hc[streams:2 * streams].float(), hc[2 * streams:].float().reshape(streams, streams)
+        new = torch.einsum("sr,tsd->trd", mix, x3.float()) + float(mult) * out[None, :, None] * yy[:, None, :]
+        xs.copy_(new.reshape(T, -1))
+        return xs
+
+    def streams_update_norm_(self, xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype):
+        """``streams_update_`` and the next sublayer's ``streams_norm`` of the new streams, in one pass."""
+        self.streams_update_(xs, y, gate, hc, mult, streams)
+        return self.streams_norm(xs, coef, w, eps, out_dtype, streams)
+
+    def scale_(self, z, alpha):
+        z.mul_(float(alpha))
+        return z
+
+    def sigmoid_gate(self, o, g, out_dtype):
+        """o * sigmoid(g), element by element."""
+        return (o.float() * torch.sigmoid(g.float())).to(out_dtype)
 
     def matmul_nt(self, a, w, bias=None, xielu=None, out_dtype=torch.float32):
         if a.dtype != w.dtype:
@@ -109,6 +155,10 @@ class TorchSeqOps:
         return self.gate_mul(gu, out_dtype, "silu")
 
     def unary(self, z, kind, out_dtype):
+        """tanh, or gelu: the exact form 0.5 z (1 + erf(z / sqrt 2))."""
+        if kind == "gelu":
+            zf = z.float()
+            return (0.5 * zf * (1.0 + torch.erf(zf * (1.0 / math.sqrt(2.0))))).to(out_dtype)
         if kind != "tanh":
             raise ValueError(kind)
         return torch.tanh(z.float()).to(out_dtype)
@@ -137,7 +187,17 @@ class TorchSeqOps:
         s = (original / wavelength - low) / (high - low)."""
         i = torch.arange(dims // 2, dtype=torch.float64)
         f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
-        if scaling is not None:
+        if scaling is not None and scaling[0] == "turns":
+            # ("turns", factor, original, fast, slow): by the entry number at which a pair makes ``fast`` /
+            # ``slow`` turns over ``original`` positions, e(t) = dims ln(original / (2 pi t)) / (2 ln base):
+            # entries up to lo = floor(e(fast)) keep their frequency, from hi = ceil(e(slow)) on they are
+            # divided by factor, a linear ramp between
+            factor, orig, fast, slow = (float(v) for v in scaling[1:])
+            e = lambda t: dims * math.log(orig / (2 * math.pi * t)) / (2 * math.log(float(base)))
+            lo, hi = max(math.floor(e(fast)), 0), min(math.ceil(e(slow)), dims - 1)
+            ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+            f = f / factor * ramp + f * (1 - ramp)
+        elif scaling is not None:
             factor, low, high, orig = (float(v) for v in scaling)
             wl = 2 * math.pi / f
             s_ = (orig / wl - low) / (high - low) if high != low else torch.ones_like(f)
@@ -145,11 +205,19 @@ class TorchSeqOps:
             f = torch.where(wl < orig / high, f, torch.where(wl > orig / low, f / factor, mid))
         return f.float().to(device)
 
+    @staticmethod
+    def rope_amp(scaling) -> float:
+        """The factor on every cosine and sine: 0.1 ln(factor) + 1 for the ("turns", ...) rescaling, else 1."""
+        if scaling is not None and scaling[0] == "turns":
+            return 0.1 * math.log(float(scaling[1])) + 1.0
+        return 1.0
+
     def head_norm_rope(self, x, heads, n, x_col, x_hs, out, out_col, out_hs, meta, w=None, eps=0.0, rot=None,
-                       row_map=None, raw=None, unit_after=False):
+                       row_map=None, raw=None, unit_after=False, half=False):
         """Per row t and head h the n entries x[t, x_col + h * x_hs : + n]: RMS-normed over n times w
         (when w is given), then the first rot = (dims, base[, scaling])[0] entries rotated in pairs
-        (2i, 2i + 1) by the angle pos_t * f_i (``rope_freqs``), then, with ``unit_after``, divided by
+        (2i, 2i + 1) -- with ``half`` in pairs (i, i + dims / 2) -- by the angle pos_t * f_i (``rope_freqs``,
+        cosine and sine times ``rope_amp``), then, with ``unit_after``, divided by
         their root mean square over n (eps inside the root, no weight); written to
         out[row, out_col + h * out_hs : + n], row = t or row_map[t].  ``raw``: a matrix like out that
         receives the entries as they came."""
@@ -160,13 +228,16 @@ class TorchSeqOps:
             v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()
         if rot is not None and rot[0] > 0:
             dims, base = rot[0], rot[1]
-            freqs = self.rope_freqs(dims, base, x.device, rot[2] if len(rot) > 2 else None)
+            sc = rot[2] if len(rot) > 2 else None
+            freqs = self.rope_freqs(dims, base, x.device, sc)
             ang = meta["tok_pos"].float()[:, None] * freqs[None, :]                                     # fp32 angles
-            c, s_ = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
-            a, b = v[:, :, 0:dims:2], v[:, :, 1:dims:2]
+            amp = self.rope_amp(sc)
+            c, s_ = amp * torch.cos(ang)[:, None, :], amp * torch.sin(ang)[:, None, :]
+            ia, ib = (slice(0, dims // 2), slice(dims // 2, dims)) if half else (slice(0, dims, 2), slice(1, dims, 2))
+            a, b = v[:, :, ia], v[:, :, ib]
             r = v.clone()
-            r[:, :, 0:dims:2] = a * c - b * s_
-            r[:, :, 1:dims:2] = b * c + a * s_
+            r[:, :, ia] = a * c - b * s_
+            r[:, :, ib] = b * c + a * s_
             v = r
         if unit_after:
             v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
@@ -214,7 +285,7 @@ class TorchSeqOps:
         vcache.view(-1, vcache.shape[-1]).index_copy_(0, kv_slot.long(), v.to(vcache.dtype))
 
     def attn_paged(self, q, kcache, vcache, meta, H, G, d, dv, scale, softcap, r1, r2, chunk, page_size, out_dtype,
-                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None, sink=None, head_gate=None):
+                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None, sink=None, head_gate=None, v_heads=None):
         """Row i of a request sees the keys j <= i of its own chunk (``chunk`` > 0: floor(i / chunk) ==
         floor(j / chunk)) or window (``window`` > 0: j > i - window, and besides them the first
         ``keep_first`` keys of the sequence), read from the request's pages.  Head h of H reads key /
@@ -222,11 +293,16 @@ class TorchSeqOps:
         the visible keys of cap(scale q.k) - r1 log(1 + r2 (i - j)), or, with ``gate_bias`` [H],
         sigmoid(scale q.k + gate_bias[h]) for each key by itself.  ``sink`` (a number): the softmax has one
         more entry of that score and no value, p_j = exp(s_j) / (exp(sink) + sum exp(s)).  ``head_gate``
-        [T, H] fp32: head h's output of row t times sigmoid(head_gate[t, h]).  The result times ``out_scale``."""
+        [T, H] fp32: head h's output of row t times sigmoid(head_gate[t, h]).  The result times ``out_scale``.
+        ``v_heads`` (a divisor of G): the pool holds only that many value heads, key head g reads value
+        head g % v_heads (several score maps over the same values).  ``out`` may be fp32 over bf16 pools."""
         T = q.shape[0]
         res = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
         kf = kcache.reshape(-1, kcache.shape[-1])[:, :G * d].reshape(-1, G, d)
-        vf = vcache.reshape(-1, vcache.shape[-1])[:, :G * dv].reshape(-1, G, dv)
+        Gv = int(v_heads or G)
+        vf = vcache.reshape(-1, vcache.shape[-1])[:, :Gv * dv].reshape(-1, Gv, dv)
+        if Gv != G:
+            vf = vf.repeat(1, G // Gv, 1)
         qf = q.float().view(T, H, d)
         pos, seq, table = meta["tok_pos"].tolist(), meta["tok_seq"].tolist(), meta["page_table"]
         rep = H // G
@@ -310,6 +386,39 @@ class TorchSeqOps:
         out.copy_(y.to(out.dtype))
         return out
 
+    def diff_combine(self, a, lam_w, diff, H, dv, eps, out_dtype):
+        """a: [T, 2 H dv], the outputs of two score maps, all heads of the first map, then all of the second.
+        Per head o = a1 - lambda a2 with lambda = exp(sum(lam_w[0] lam_w[1])) - exp(sum(lam_w[2] lam_w[3])) + diff,
+        then o / sqrt(mean(o^2) + eps) * (1 - diff)."""
+        T = a.shape[0]
+        lw = lam_w.float()
+        lam = torch.exp((lw[0] * lw[1]).sum()) - torch.exp((lw[2] * lw[3]).sum()) + float(diff)
+        a3 = a.float().reshape(T, 2, H, dv)
+        o = a3[:, 0] - lam * a3[:, 1]
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * (1.0 - float(diff))
+        return o.reshape(T, H * dv).to(out_dtype)
+
+    def hgrn2_scan(self, q, f, v, fb, lower, norm_w, state, meta, heads, dim, vdim, eps, out_dtype):
+        """Per head a state S [dim, vdim] carried in ``state[slot]``: with the forget gate
+        g_t = lower + (1 - lower) sigmoid(f_t + fb) per state row,  S_t = diag(g_t) S_(t-1) + (1 - g_t) v_t^T,
+        o_t = S_t^T silu(q_t); returns o / sqrt(mean_head(o^2) + eps) * norm_w (norm_w [vdim], shared by the heads)."""
+        T, H = q.shape[0], heads
+        qq = F.silu(q.float()).reshape(T, H, dim)
+        lo = lower.float()
+        ff = f.float() + fb.float() if fb is not None else f.float()      # (fb None: the bias is already in f)
+        gg = (lo + (1 - lo) * torch.sigmoid(ff)).reshape(T, H, dim)
+        vv = v.float().reshape(T, H, vdim)
+        o = torch.empty(T, H, vdim, dtype=torch.float32, device=q.device)
+        cu, pos0, slot = meta["cu_host"], meta["pos0_host"], meta["slot"].tolist()
+        for s in range(len(slot)):
+            S = state[slot[s]].clone() if pos0[s] > 0 else torch.zeros(H, dim, vdim, device=q.device)
+            for t in range(int(cu[s]), int(cu[s + 1])):
+                S = gg[t][:, :, None] * S + (1 - gg[t])[:, :, None] * vv[t][:, None, :]
+                o[t] = torch.einsum("hkv,hk->hv", S, qq[t])
+            state[slot[s]] = S
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+        return o.reshape(T, H * vdim).to(out_dtype)
+
     def rglru_scan(self, u, g, lam, y, state, meta, c, out_dtype):
         """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) sigmoid(g_i) u_t,  a_t = exp(-c sigmoid(g_r) softplus(lam));
         returns S_t * gelu_tanh(y_t)."""
@@ -373,6 +482,32 @@ class TorchSeqOps:
         T, E = logits.shape
         vals, ids = torch.sort(logits.float(), dim=-1, descending=True, stable=True)
         ids, w = ids[:, :top], torch.softmax(vals[:, :top], -1)
+        flat = ids.reshape(-1)
+        order = torch.sort(flat, stable=True).indices
+        dest = torch.empty_like(order)
+        dest[order] = torch.arange(order.numel(), device=order.device)
+        offs = torch.zeros(E + 1, dtype=torch.int32, device=logits.device)
+        offs[1:] = torch.cumsum(torch.bincount(flat, minlength=E), 0)
+        return SeqRoute(ids.int(), w, offs, (order // top).int(), dest.int().reshape(T, top), top)
+
+    def moe_route_grouped(self, logits, top, groups, keep, scale):
+        """Scores sigmoid(logit).  The experts form ``groups`` equal groups of neighbours, a group is worth the
+        sum of its two largest scores, and only experts of the ``keep`` best groups compete (``groups`` 0 or
+        1: all do).  The ``top`` largest scores are chosen (ties: the lower expert), weighted by
+        score / (sum of the chosen + 1e-20) * scale."""
+        T, E = logits.shape
+        sc = torch.sigmoid(logits.float())
+        cand = sc
+        if groups and groups > 1:
+            per = E // groups
+            worth = torch.sort(sc.reshape(T, groups, per), dim=-1, descending=True).values[:, :, :2].sum(-1)
+            kept = torch.sort(worth, dim=-1, descending=True, stable=True).indices[:, :keep]
+            ok = torch.zeros(T, groups, dtype=torch.bool, device=logits.device)
+            ok.scatter_(1, kept, True)
+            cand = torch.where(ok.repeat_interleave(per, 1), sc, torch.full_like(sc, -1.0))
+        ids = torch.sort(cand, dim=-1, descending=True, stable=True).indices[:, :top]
+        w = sc.gather(1, ids)
+        w = w / (w.sum(-1, keepdim=True) + 1e-20) * float(scale)
         flat = ids.reshape(-1)
         order = torch.sort(flat, stable=True).indices
         dest = torch.empty_like(order)

@@ -40,7 +40,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from ..models.layout import ALIGN_BYTES, layer_kind
+from ..models.layout import ALIGN_BYTES, layer_image, layer_kind
 from . import hostmem
 from .weights import LayerSource
 
@@ -148,8 +148,12 @@ class ShardPrefetcher:
         self.lock = threading.Lock()
 
     # ------------------------------------------------------------ helpers
+    def _images(self, k: int) -> List[str]:
+        """The distinct weight images of shard k (passes of a looped layer share one), in order."""
+        return list(dict.fromkeys(layer_image(self.names[i]) for i in self.shards[k]))
+
     def shard_bytes(self, k: int) -> int:
-        return sum(_align(self.src.nbytes(self.names[i])) for i in self.shards[k])
+        return sum(_align(self.src.nbytes(n)) for n in self._images(k))
 
     def slot_of(self, k: int, epoch: Optional[int] = None) -> int:
         if self.resident or self._big_idx[k] < 0:
@@ -191,14 +195,18 @@ class ShardPrefetcher:
         t0 = time.perf_counter()
         s = self.slot_of(k, epoch)
         views: Dict[str, Dict[str, torch.Tensor]] = {}
+        by_image: Dict[str, Dict[str, torch.Tensor]] = {}      # passes of a looped layer in one shard: one copy
         if not self.cuda:
             for i in self.shards[k]:
                 name = self.names[i]
+                if layer_image(name) in by_image:
+                    views[name] = by_image[layer_image(name)]
+                    continue
                 hb = self.src.host_buffer(name)
                 if hb is None:
                     hb = torch.empty(self.src.nbytes(name), dtype=torch.uint8)
                     self.src.read_into(name, hb)
-                views[name] = self.src.layout(name).views(hb, self.dtype)
+                views[name] = by_image[layer_image(name)] = self.src.layout(name).views(hb, self.dtype)
             self.load_seconds += time.perf_counter() - t0
             return None, views, s
         slot = self._slot(s)
@@ -209,6 +217,9 @@ class ShardPrefetcher:
             off = 0
             for i in self.shards[k]:
                 name = self.names[i]
+                if layer_image(name) in by_image:
+                    views[name] = by_image[layer_image(name)]
+                    continue
                 nb = self.src.nbytes(name)
                 dst = slot[off:off + nb]
                 hb = self.src.host_buffer(name)
@@ -223,7 +234,7 @@ class ShardPrefetcher:
                     self._staging_ev[si] = e
                 else:
                     dst.copy_(hb[:nb], non_blocking=True)
-                views[name] = self.src.layout(name).views(dst, self.dtype)
+                views[name] = by_image[layer_image(name)] = self.src.layout(name).views(dst, self.dtype)
                 self._loaded(name, views[name])
                 off += _align(nb)
                 self.bytes_h2d += nb

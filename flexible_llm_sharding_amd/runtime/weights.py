@@ -28,7 +28,7 @@ from typing import Dict, List, NamedTuple, Optional, Sequence, Tuple
 import torch
 
 from ..config import ModelConfig
-from ..models.layout import LayerLayout, layer_kind, layer_layout, layer_layout_of
+from ..models.layout import LayerLayout, layer_image, layer_kind, layer_layout, layer_layout_of
 from . import hostmem
 
 
@@ -100,6 +100,10 @@ class HostStore(LayerSource):
         dst[:src.numel()].copy_(src)
 
     def alloc(self, name: str) -> torch.Tensor:
+        for other, buf in self.buffers.items():         # a later pass of a looped layer: the same image
+            if other != name and layer_image(other) == layer_image(name):
+                self.buffers[name] = buf
+                return buf
         buf = hostmem.alloc_host(self.nbytes(name), pinned=self.pinned)
         self.buffers[name] = buf
         return buf
@@ -111,7 +115,7 @@ class HostStore(LayerSource):
         for n in st.names:
             st.alloc(n)
         errs: List[BaseException] = []
-        todo = list(st.names)
+        todo = list({layer_image(n): n for n in reversed(st.names)}.values())[::-1]      # one read per image
         lock = threading.Lock()
 
         def worker():
