@@ -40,16 +40,18 @@ int fls_seq_gather_rows(const void* x, int tx, int ldx, const int* idx, void* y,
 int fls_seq_xielu(const float* z, int ldz, const float* act, void* y, int ty, int ldy, int rows, int cols, fls_stream_t s);
 // y[r, c] = act(gu[r, c]) * gu[r, cols + c]; act: 0 = silu, 1 = gelu (tanh form)
 int fls_seq_gate_mul(const float* gu, int ldg, void* y, int ty, int ldy, int rows, int cols, int act, fls_stream_t s);
-// y = f(z) elementwise; kind: 0 = tanh
+// y = f(z) elementwise; kind: 0 = tanh, 1 = gelu (exact: 0.5 z (1 + erf(z / sqrt 2)))
 int fls_seq_unary(const float* z, int ldz, void* y, int ty, int ldy, int rows, int cols, int kind, fls_stream_t s);
 // per row t and head h: the n entries x[t, x_col + h x_hs ...] (x of type tx), RMS-normed over n times w[n] (w != null), the first
 // rot entries rotated in pairs (2i, 2i+1) by the angle tok_pos[t] * freqs[i]; written as type to at
 // out[row, out_col + h out_hs ...], row = row_map ? row_map[t] : t; raw (nullable, like out, row stride ldr)
 // receives the entries unchanged.  unit_after != 0: after the rotation the n entries are divided by
-// sqrt(mean(entries^2) + eps), without a weight.  n <= 512
+// sqrt(mean(entries^2) + eps), without a weight.  n <= 512.  half != 0: the pairs are (i, i + rot / 2) instead;
+// amp: a factor on every cosine and sine
 int fls_seq_head_norm_rope(const void* x, int tx, int ldx, int x_col, int x_hs, int heads, int n, const float* w, float eps,
                            const float* freqs, int rot, const int* tok_pos, const int* row_map, void* out, int to,
-                           int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, int unit_after, fls_stream_t s);
+                           int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, int unit_after, int half, float amp,
+                           fls_stream_t s);
 int fls_seq_softcap(float* z, int ldz, int rows, int cols, float cap, fls_stream_t s);
 int fls_seq_argmax(const float* z, int ldz, int rows, int cols, int* out, fls_stream_t s);
 // k rows RMS-normed over all kcols (times kn), k and v rows written at row kv_slot[r] of the pools
@@ -66,21 +68,23 @@ int fls_seq_kv_store(const float* k, int ldk, const float* kn, float eps, const 
 // kernel; part: T H nsplit (dv + 4) floats of scratch (16-byte aligned).  has_sink != 0 (softmax only): one more
 // entry of score `sink` and no value joins the softmax's sum.  head_gate (nullable) [T, H] fp32, row stride ldhg:
 // the output of (row, head) times sigmoid(head_gate[t, h]).
+// out of type to (fp32 over bf16 pools allowed).  Gv (0: G), a divisor of G: the value pool holds Gv heads and key head g
+// reads value head g % Gv (several score maps over the same values).
 int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, int tc,
-                       void* out, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
+                       void* out, int to, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
                        int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
                        const float* r1, const float* r2, int chunk, int window, int keep_first,
                        const float* gate_bias, float out_scale, int page_size, int nsplit, float* part,
-                       int has_sink, float sink, const float* head_gate, int ldhg, fls_stream_t s);
+                       int has_sink, float sink, const float* head_gate, int ldhg, int Gv, fls_stream_t s);
 // the same attention on the matrix cores for bf16 pools and rows in tiles: tiles[n_tiles][2] = (first packed
 // row, rows <= 128) of one request each, covering every row of the step; q of type tq.  -2: shape not
 // served (use the above)
 int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, void* out,
-                         int ldo, const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
+                         int to, int ldo, const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
                          const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
                          float softcap, const float* r1, const float* r2, int chunk, int window, int keep_first,
                          const float* gate_bias, float out_scale, int page_size, int has_sink, float sink,
-                         const float* head_gate, int ldhg, fls_stream_t s);
+                         const float* head_gate, int ldhg, int Gv, fls_stream_t s);
 // softmax attention of few rows whose H / G <= 32 query heads per key / value head become the columns of one
 // matrix-core tile (decode steps over cached latent rows): fp32 q, bf16 pools and out, window and kept first
 // keys as above; nsplit ranges of key tiles per row, part: T H nsplit (dv + 4) floats.  -2: shape not served
@@ -136,6 +140,11 @@ int fls_seq_ssd_scan(const float* xbc, int ldx, const float* z, int ldz, const f
 // corr == null: the top largest logits are chosen and w = the softmax over the chosen logits only
 int fls_seq_moe_route(const float* logits, int ldl, const float* corr, int T, int E, int top, int* ids, float* w,
                       int* hist, fls_stream_t s);
+// scores sigmoid(logit); `groups` equal groups of neighbouring experts, each worth the sum of its two largest scores;
+// only experts of the `keep` best groups compete (groups <= 1: all); the top largest scores are chosen (ties: the
+// lower expert), w = score / (sum of the chosen + 1e-20) * scale; hist as above.  groups <= 64
+int fls_seq_moe_route_grouped(const float* logits, int ldl, int T, int E, int top, int groups, int keep, float scale,
+                              int* ids, float* w, int* hist, fls_stream_t s);
 // offs[E+1] = exclusive scan of hist; cursor[E] = offs[:E]
 int fls_seq_moe_scan(const int* hist, int E, int* offs, int* cursor, fls_stream_t s);
 // dest[t, k] = a row in its expert's range; rows[dest] = t
@@ -146,6 +155,33 @@ int fls_seq_moe_sum(const float* y, int ldy, const int* dest, const float* w, fl
 // x[t] += mult * (sum_k w[t, k] y[dest[t, k]] + sigmoid(gate[t * ldg]) shared[t]); shared nullable, gate nullable (then 1)
 int fls_seq_moe_combine(float* x, int ldx, const float* y, int ldy, const int* dest, const float* w, int T, int top,
                         const float* shared, int lds, const float* gate, int ldg, int D, float mult, fls_stream_t s);
+// ---- several residual streams per row (streams.hip).  xs: fp32 [rows, S D], a row's S streams side by side
+// out[t, c * D ...] = table[ids[t]] * scale + pos_table[tok_pos[t]] (pos_table nullable; positions clamped to P - 1), c < copies
+int fls_seq_embed_pos(const int* ids, const void* table, int tt, const void* pos_table, const int* tok_pos, float* out, int T,
+                      int D, int V, int P, float scale, int copies, fls_stream_t s);
+// u = sum_s coef[s] xs[row, s] (coef nullable: the plain sum), y[r] = u / sqrt(mean(u^2) + eps) * w; row = idx ? idx[r] : r
+int fls_seq_streams_norm(const float* xs, int ldx, const int* idx, const float* coef, const float* w, void* y, int ty, int ldy,
+                         int rows, int D, int S, float eps, fls_stream_t s);
+// all streams at once from the old ones: xs[t, r] <- sum_s mix[s, r] xs[t, s] + mult * out[r] * y[t] * sigmoid(gate[t]);
+// hc = [in (S) | out (S) | mix (S x S, [from, to])] (nullable: S = 1, out = mix = 1); gate nullable.  h != null: also
+// h[t] = the norm above of the NEW streams with coefficients ncoef (nullable) and weight nw, type th
+int fls_seq_streams_update(float* xs, int ldx, const float* y, int ldy, const float* gate, int ldg, const float* hc, float mult,
+                           int rows, int D, int S, const float* ncoef, const float* nw, void* h, int th, int ldh, float eps,
+                           fls_stream_t s);
+int fls_seq_scale(float* z, int ldz, int rows, int cols, float alpha, fls_stream_t s);
+// y = o * sigmoid(g); o of type to_, y of type ty
+int fls_seq_sigmoid_gate(const void* o, int to_, int ldo, const float* g, int ldg, void* y, int ty, int ldy, int rows, int cols,
+                         fls_stream_t s);
+// a: fp32 [T, 2 H dv], two score maps' outputs (all heads of map 1, then of map 2); per head o = a1 - lambda a2,
+// lambda = exp(sum(lam_w[0] lam_w[1])) - exp(sum(lam_w[2] lam_w[3])) + diff (lam_w: [4, d]); out = o / sqrt(mean(o^2) + eps) (1 - diff)
+int fls_seq_diff_combine(const float* a, int lda, const float* lam_w, int d, float diff, int H, int dv, float eps, void* out,
+                         int to, int ldo, int T, fls_stream_t s);
+// HGRN2, per head a state S[d][dv] in state[slot][H][d][dv]: g = lower + (1 - lower) sigmoid(f (+ fb)),
+// S_t = diag(g_t) S_(t-1) + (1 - g_t) v_t^T, o_t = S_t^T silu(q_t); raw: fp32 [T, H dv] (row stride ldo), o before its norm.
+// q, f: fp32 [T, H d], v: fp32 [T, H dv] with their row strides; fb nullable; d <= 256
+int fls_seq_hgrn2_scan(const float* q, int ldq, const float* f, int ldf, const float* v, int ldv, const float* fb,
+                       const float* lower, float* state, float* raw, int ldo, const int* cu, const int* pos0,
+                       const int* slot, int B, int H, int d, int dv, fls_stream_t s);
 #ifdef __cplusplus
 }
 #endif

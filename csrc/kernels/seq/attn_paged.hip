@@ -49,9 +49,9 @@ __device__ __forceinline__ float dot_row(const T* __restrict__ k, const float* _
   return acc;
 }
 
-template <typename TQ, typename T>
+template <typename TQ, typename T, typename TO>
 __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ q, int ldq, const T* kc, int ldk,
-                                                         const T* vc, int ldv, T* __restrict__ out, int ldo,
+                                                         const T* vc, int ldv, TO* __restrict__ out, int ldo,
                                                          const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                                          const int* __restrict__ page_table, int pt_stride, int H, int G,
                                                          int d, int dv, float scale, float softcap,
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
                                                          int chunk, int window, int keep_first,
                                                          const float* __restrict__ gate_bias, float out_scale,
                                                          int page_size, int vec, float* __restrict__ part, int has_sink,
-                                                         float sink, const float* __restrict__ head_gate, int ldhg) {
+                                                         float sink, const float* __restrict__ head_gate, int ldhg, int Gv) {
   __shared__ float qs[MAX_D];
   __shared__ float pw[4][64];
   __shared__ int prow[4][64];
@@ -67,6 +67,7 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
   __shared__ float accs[4][MAX_DV_PER_LANE * 64];
   const int t = blockIdx.y, h = blockIdx.x;
   const int g = h / (H / G);
+  const int gv = g % Gv;                          // (several score maps over the same values: Gv < G value heads)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int i = tok_pos[t];
   const int* table = page_table + (size_t)tok_seq[t] * pt_stride;
@@ -127,11 +128,11 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(const TQ* __restrict__ 
         for (; jj + 8 <= nk; jj += 8) {            // eight independent value loads in flight
           float v[8];
 #pragma unroll
-          for (int x = 0; x < 8; ++x) v[x] = ldf(vc + (size_t)prow[wave][jj + x] * ldv + (size_t)g * dv, e);
+          for (int x = 0; x < 8; ++x) v[x] = ldf(vc + (size_t)prow[wave][jj + x] * ldv + (size_t)gv * dv, e);
 #pragma unroll
           for (int x = 0; x < 8; ++x) a += pw[wave][jj + x] * v[x];
         }
-        for (; jj < nk; ++jj) a += pw[wave][jj] * ldf(vc + (size_t)prow[wave][jj] * ldv + (size_t)g * dv, e);
+        for (; jj < nk; ++jj) a += pw[wave][jj] * ldf(vc + (size_t)prow[wave][jj] * ldv + (size_t)gv * dv, e);
         acc[c] = a;
       }
     }
@@ -218,35 +219,45 @@ int seq_attn_merge(const float* part, void* out, int tc, int ldo, int T, int H, 
   return 0;
 }
 
-// tq: type of q; tc: type of the pools and of out
+// tq: type of q; tc: type of the pools; to: type of out (fp32 over bf16 pools allowed)
 extern "C" int fls_seq_attn_paged(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, int tc,
-                                  void* out, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
+                                  void* out, int to, int ldo, const int* tok_seq, const int* tok_pos, const int* page_table,
                                   int pt_stride, int T, int H, int G, int d, int dv, float scale, float softcap,
                                   const float* r1, const float* r2, int chunk, int window, int keep_first,
                                   const float* gate_bias, float out_scale, int page_size, int nsplit, float* part,
-                                  int has_sink, float sink, const float* head_gate, int ldhg, fls_stream_t s) {
+                                  int has_sink, float sink, const float* head_gate, int ldhg, int Gv, fls_stream_t s) {
   if (T <= 0) return 0;
+  if (Gv <= 0) Gv = G;
+  if (G % Gv || (to == 1 && tc == 0)) return -1;
   if (has_sink && gate_bias != nullptr) return -1;      // (a silent entry belongs to a softmax)
   if (nsplit < 1 || nsplit > MERGE_MAX_SPLIT || (nsplit > 1 && part == nullptr)) return -1;
-  if (d > MAX_D || dv > 64 * MAX_DV_PER_LANE || G < 1 || H % G || page_size < 1 || G * d > ldk || G * dv > ldv || keep_first < 0
+  if (d > MAX_D || dv > 64 * MAX_DV_PER_LANE || G < 1 || H % G || page_size < 1 || G * d > ldk || Gv * dv > ldv || keep_first < 0
       || (tq == 1 && tc == 0)) return -1;
   dim3 grid(H, T, nsplit);
   hipStream_t st = (hipStream_t)s;
-#define ATTN_PAGED_ARGS ldq, (const TC*)kc, ldk, (const TC*)vc, ldv, (TC*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, \
+#define ATTN_PAGED_ARGS ldq, (const TC*)kc, ldk, (const TC*)vc, ldv, (TOUT*)out, ldo, tok_seq, tok_pos, page_table, pt_stride, H, G, \
                         d, dv, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias, out_scale, page_size, vec, part, has_sink, sink, \
-                        nsplit > 1 ? nullptr : head_gate, ldhg
+                        nsplit > 1 ? nullptr : head_gate, ldhg, Gv
   if (tc == 1) {
     using TC = bf16_t;
     const int vec = d % 8 == 0 && (uintptr_t)kc % 16 == 0 && ldk % 8 == 0;
-    if (tq == 1) hipLaunchKernelGGL((attn_paged_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, st, (const bf16_t*)q, ATTN_PAGED_ARGS);
-    else hipLaunchKernelGGL((attn_paged_kernel<float, bf16_t>), grid, dim3(256), 0, st, (const float*)q, ATTN_PAGED_ARGS);
+    if (to == 0) {
+      using TOUT = float;
+      if (tq == 1) hipLaunchKernelGGL((attn_paged_kernel<bf16_t, bf16_t, float>), grid, dim3(256), 0, st, (const bf16_t*)q, ATTN_PAGED_ARGS);
+      else hipLaunchKernelGGL((attn_paged_kernel<float, bf16_t, float>), grid, dim3(256), 0, st, (const float*)q, ATTN_PAGED_ARGS);
+    } else {
+      using TOUT = bf16_t;
+      if (tq == 1) hipLaunchKernelGGL((attn_paged_kernel<bf16_t, bf16_t, bf16_t>), grid, dim3(256), 0, st, (const bf16_t*)q, ATTN_PAGED_ARGS);
+      else hipLaunchKernelGGL((attn_paged_kernel<float, bf16_t, bf16_t>), grid, dim3(256), 0, st, (const float*)q, ATTN_PAGED_ARGS);
+    }
   } else {
     using TC = float;
+    using TOUT = float;
     const int vec = d % 4 == 0 && (uintptr_t)kc % 16 == 0 && ldk % 4 == 0;
-    hipLaunchKernelGGL((attn_paged_kernel<float, float>), grid, dim3(256), 0, st, (const float*)q, ATTN_PAGED_ARGS);
+    hipLaunchKernelGGL((attn_paged_kernel<float, float, float>), grid, dim3(256), 0, st, (const float*)q, ATTN_PAGED_ARGS);
   }
 #undef ATTN_PAGED_ARGS
   SEQ_LAUNCH_CHECK();
-  if (nsplit > 1) return seq_attn_merge(part, out, tc, ldo, T, H, dv, nsplit, gate_bias != nullptr, out_scale, has_sink, sink, head_gate, ldhg, s);
+  if (nsplit > 1) return seq_attn_merge(part, out, to, ldo, T, H, dv, nsplit, gate_bias != nullptr, out_scale, has_sink, sink, head_gate, ldhg, s);
   return 0;
 }

@@ -27,9 +27,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 #define KT 32             // keys per tile
 #define PLD (KT + 8)      // row stride (elements) of the transposed V tile and of the weight tiles
 
-template <int D, int DV, typename TQ>
+template <int D, int DV, typename TQ, typename TO>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const TQ* __restrict__ q, int ldq, const bf16_t* __restrict__ kc, int ldk,
-                                                           const bf16_t* __restrict__ vc, int ldv, bf16_t* __restrict__ out, int ldo,
+                                                           const bf16_t* __restrict__ vc, int ldv, TO* __restrict__ out, int ldo,
                                                            const int* __restrict__ tiles, const int* __restrict__ tok_seq,
                                                            const int* __restrict__ tok_pos, const int* __restrict__ page_table,
                                                            int pt_stride, int H, int G, float scale, float softcap,
@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const TQ* __restrict_
                                                            int chunk, int window, int keep_first,
                                                            const float* __restrict__ gate_bias, float out_scale, int page_size,
                                                            int has_sink, float sink, const float* __restrict__ head_gate,
-                                                           int ldhg) {
+                                                           int ldhg, int Gv) {
   constexpr int KLD = D + 8;
   __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t Vt[DV * PLD];
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const TQ* __restrict_
       vreg[x] = make_uint4(0, 0, 0, 0);
       if (j < jend) {
         const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
-        vreg[x] = *reinterpret_cast<const uint4*>(vc + row * ldv + (size_t)g * DV + seg * 8);
+        vreg[x] = *reinterpret_cast<const uint4*>(vc + row * ldv + (size_t)(g % Gv) * DV + seg * 8);
       }
     }
   };
@@ -218,47 +218,52 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const TQ* __restrict_
   if (qok && (gated || l > 0.f)) {
     float inv = gated ? out_scale : out_scale / l;
     if (head_gate != nullptr) inv *= sigmoid_f(head_gate[(size_t)(row0 + qrow) * ldhg + h]);
-    bf16_t* op = out + (size_t)(row0 + qrow) * ldo + (size_t)h * DV;
+    TO* op = out + (size_t)(row0 + qrow) * ldo + (size_t)h * DV;
 #pragma unroll
     for (int c = 0; c < DV / 32; ++c)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        bf16_t o4[4];
+        if constexpr (sizeof(TO) == 4) {
+          *reinterpret_cast<float4*>(op + 32 * c + 8 * rg + 4 * h2) =
+              make_float4(O[c][4 * rg] * inv, O[c][4 * rg + 1] * inv, O[c][4 * rg + 2] * inv, O[c][4 * rg + 3] * inv);
+        } else {
+          bf16_t o4[4];
 #pragma unroll
-        for (int x = 0; x < 4; ++x) o4[x] = f_to_bf16(O[c][4 * rg + x] * inv);
-        *reinterpret_cast<uint2*>(op + 32 * c + 8 * rg + 4 * h2) = *reinterpret_cast<const uint2*>(o4);
+          for (int x = 0; x < 4; ++x) o4[x] = f_to_bf16(O[c][4 * rg + x] * inv);
+          *reinterpret_cast<uint2*>(op + 32 * c + 8 * rg + 4 * h2) = *reinterpret_cast<const uint2*>(o4);
+        }
       }
   }
 }
 
 // tiles: n_tiles x (first packed row, rows <= 128) of one request each.  tq: type of q (0 fp32, 1 bf16);
-// pools and out are bf16.  Returns -2 for head sizes or alignments this kernel does not serve (the
+// pools are bf16, out of type to.  Gv (0: G): value heads in the pool, key head g reads value head g % Gv.  Returns -2 for head sizes or alignments this kernel does not serve (the
 // caller then runs fls_seq_attn_paged).
 extern "C" int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* kc, int ldk, const void* vc, int ldv, void* out,
-                                    int ldo, const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
+                                    int to, int ldo, const int* tiles, int n_tiles, const int* tok_seq, const int* tok_pos,
                                     const int* page_table, int pt_stride, int H, int G, int d, int dv, float scale,
                                     float softcap, const float* r1, const float* r2, int chunk, int window, int keep_first,
                                     const float* gate_bias, float out_scale, int page_size, int has_sink, float sink,
-                                    const float* head_gate, int ldhg, fls_stream_t s) {
+                                    const float* head_gate, int ldhg, int Gv, fls_stream_t s) {
   if (n_tiles <= 0) return 0;
   if (has_sink && gate_bias != nullptr) return -1;
-  if (G < 1 || H % G || page_size < 1 || ldq % 8 || ldo % 4 || ldk % 8 || ldv % 8 || G * d > ldk || G * dv > ldv ||
-      (uintptr_t)q % 16 || (uintptr_t)kc % 16 || (uintptr_t)vc % 16 || (uintptr_t)out % 8 || keep_first < 0)
+  if (Gv <= 0) Gv = G;
+  if (G < 1 || H % G || G % Gv || page_size < 1 || ldq % 8 || ldo % 4 || ldk % 8 || ldv % 8 || G * d > ldk || Gv * dv > ldv ||
+      (uintptr_t)q % 16 || (uintptr_t)kc % 16 || (uintptr_t)vc % 16 || (uintptr_t)out % 16 || keep_first < 0)
     return -2;
   dim3 grid(H, n_tiles);
   hipStream_t st = (hipStream_t)s;
+#define ATTN_PF_(DD, DDV, TQ_, TO_)                                                                                       \
+  hipLaunchKernelGGL((attn_prefill_kernel<DD, DDV, TQ_, TO_>), grid, dim3(256), 0, st, (const TQ_*)q, ldq,                \
+                     (const bf16_t*)kc, ldk, (const bf16_t*)vc, ldv, (TO_*)out, ldo, tiles, tok_seq, tok_pos,             \
+                     page_table, pt_stride, H, G, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias,           \
+                     out_scale, page_size, has_sink, sink, head_gate, ldhg, Gv)
 #define ATTN_PF(DD, DDV)                                                                                                  \
   do {                                                                                                                    \
-    if (tq == 1)                                                                                                          \
-      hipLaunchKernelGGL((attn_prefill_kernel<DD, DDV, bf16_t>), grid, dim3(256), 0, st, (const bf16_t*)q, ldq,           \
-                         (const bf16_t*)kc, ldk, (const bf16_t*)vc, ldv, (bf16_t*)out, ldo, tiles, tok_seq, tok_pos,      \
-                         page_table, pt_stride, H, G, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias,       \
-                         out_scale, page_size, has_sink, sink, head_gate, ldhg);                                          \
-    else                                                                                                                  \
-      hipLaunchKernelGGL((attn_prefill_kernel<DD, DDV, float>), grid, dim3(256), 0, st, (const float*)q, ldq,             \
-                         (const bf16_t*)kc, ldk, (const bf16_t*)vc, ldv, (bf16_t*)out, ldo, tiles, tok_seq, tok_pos,      \
-                         page_table, pt_stride, H, G, scale, softcap, r1, r2, chunk, window, keep_first, gate_bias,       \
-                         out_scale, page_size, has_sink, sink, head_gate, ldhg);                                          \
+    if (tq == 1 && to == 1) ATTN_PF_(DD, DDV, bf16_t, bf16_t);                                                            \
+    else if (tq == 1) ATTN_PF_(DD, DDV, bf16_t, float);                                                                   \
+    else if (to == 1) ATTN_PF_(DD, DDV, float, bf16_t);                                                                   \
+    else ATTN_PF_(DD, DDV, float, float);                                                                                 \
   } while (0)
   if (d == 128 && dv == 128) ATTN_PF(128, 128);
   else if (d == 64 && dv == 64) ATTN_PF(64, 64);
@@ -266,6 +271,7 @@ extern "C" int fls_seq_attn_prefill(const void* q, int ldq, int tq, const void* 
   else if (d == 64 && dv == 128) ATTN_PF(64, 128);
   else return -2;
 #undef ATTN_PF
+#undef ATTN_PF_
   SEQ_LAUNCH_CHECK();
   return 0;
 }

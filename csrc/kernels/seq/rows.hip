@@ -235,17 +235,21 @@ extern "C" int fls_seq_gate_mul(const float* gu, int ldg, void* y, int ty, int l
   return 0;
 }
 
-// y = f(z) elementwise; kind: 0 = tanh
+// y = f(z) elementwise; kind: 0 = tanh, 1 = gelu in its exact form 0.5 z (1 + erf(z / sqrt 2))
 template <typename TO>
 __global__ void unary_kernel(const float* __restrict__ z, int ldz, TO* __restrict__ y, int ldy, int cols, int kind) {
   const float* zr = z + (size_t)blockIdx.x * ldz;
   TO* yr = y + (size_t)blockIdx.x * ldy;
+  if (kind == 1) {
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) { const float v = zr[c]; stf(yr, c, 0.5f * v * (1.f + erff(v * 0.70710678118654752f))); }
+    return;
+  }
   for (int c = threadIdx.x; c < cols; c += blockDim.x) stf(yr, c, tanhf(zr[c]));
 }
 
 extern "C" int fls_seq_unary(const float* z, int ldz, void* y, int ty, int ldy, int rows, int cols, int kind, fls_stream_t s) {
   if (rows <= 0) return 0;
-  if (kind != 0) return -1;
+  if (kind != 0 && kind != 1) return -1;
   if (ty == 1) hipLaunchKernelGGL((unary_kernel<bf16_t>), dim3(rows), dim3(256), 0, (hipStream_t)s, z, ldz, (bf16_t*)y, ldy, cols, kind);
   else hipLaunchKernelGGL((unary_kernel<float>), dim3(rows), dim3(256), 0, (hipStream_t)s, z, ldz, (float*)y, ldy, cols, kind);
   SEQ_LAUNCH_CHECK();
@@ -336,7 +340,7 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(const TI* x, int ld
                                                              const float* __restrict__ freqs, int rot,
                                                              const int* __restrict__ tok_pos, const int* __restrict__ row_map,
                                                              TO* out, int ldo, int out_col, int out_hs, TO* raw, int ldr,
-                                                             int items, int unit_after) {
+                                                             int items, int unit_after, int half, float amp) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (item >= items) return;
@@ -356,22 +360,38 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(const TI* x, int ld
 #pragma unroll
     for (int e = 0; e < HNR_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) stf(rr, c, v[e]); }
   }
+  float rs_w = 1.f;
   if (w != nullptr) {
     const float rs = 1.f / sqrtf(wave_sum(ss) / (float)n + eps);
+    rs_w = rs;
 #pragma unroll
     for (int e = 0; e < HNR_MAX_E; ++e) { const int c = lane + 64 * e; if (c < n) v[e] *= rs * w[c]; }
   }
   const float pos = rot > 0 ? (float)tok_pos[t] : 0.f;
   TO* orow = out + row * ldo + out_col + (size_t)h * out_hs;
+  // the pair's other entry: in the neighbouring lane for pairs (2i, 2i + 1); for pairs (i, i + rot / 2) it is read
+  // from the row again and normed alike (all of them before anything is stored: out may be x)
+  float oth[HNR_MAX_E];
+  const int hr = rot >> 1;
 #pragma unroll
   for (int e = 0; e < HNR_MAX_E; ++e) {
     const int c = lane + 64 * e;
-    const float other = __shfl_xor(v[e], 1, 64);       // the pair's other entry sits in the neighbouring lane
+    oth[e] = __shfl_xor(v[e], 1, 64);
+    if (half && c < rot) {
+      const int pc = c >= hr ? c - hr : c + hr;
+      oth[e] = ldf(xr, pc) * (w != nullptr ? rs_w * w[pc] : 1.f);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < HNR_MAX_E; ++e) {
+    const int c = lane + 64 * e;
     float val = v[e];
     if (c < rot) {
-      const float ang = pos * freqs[c >> 1];
-      const float cs = cosf(ang), sn = sinf(ang);
-      val = (c & 1) ? v[e] * cs + other * sn : v[e] * cs - other * sn;
+      const bool second = half ? c >= hr : (c & 1);
+      const int fi = half ? (second ? c - hr : c) : (c >> 1);
+      const float ang = pos * freqs[fi];
+      const float cs = amp * cosf(ang), sn = amp * sinf(ang);
+      val = second ? v[e] * cs + oth[e] * sn : v[e] * cs - oth[e] * sn;
     }
     if (!unit_after) { if (c < n) stf(orow, c, val); }
     else v[e] = val;
@@ -389,14 +409,14 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(const TI* x, int ld
 extern "C" int fls_seq_head_norm_rope(const void* x, int tx, int ldx, int x_col, int x_hs, int heads, int n, const float* w,
                                       float eps, const float* freqs, int rot, const int* tok_pos, const int* row_map, void* out,
                                       int to, int ldo, int out_col, int out_hs, void* raw, int ldr, int rows, int unit_after,
-                                      fls_stream_t s) {
+                                      int half, float amp, fls_stream_t s) {
   if (rows <= 0 || heads <= 0) return 0;
   if (n < 1 || n > 64 * HNR_MAX_E || rot < 0 || rot > n || (rot & 1) || (rot > 0 && (freqs == nullptr || tok_pos == nullptr))) return -1;
   const int items = rows * heads;
   dim3 grid((items + 3) / 4);
   hipStream_t st = (hipStream_t)s;
 #define HNR(TI, TO) hipLaunchKernelGGL((head_norm_rope_kernel<TI, TO>), grid, dim3(256), 0, st, (const TI*)x, ldx, x_col, x_hs, heads, \
-                                       n, w, eps, freqs, rot, tok_pos, row_map, (TO*)out, ldo, out_col, out_hs, (TO*)raw, ldr, items, unit_after)
+                                       n, w, eps, freqs, rot, tok_pos, row_map, (TO*)out, ldo, out_col, out_hs, (TO*)raw, ldr, items, unit_after, half, amp)
   if (tx == 1 && to == 1) HNR(bf16_t, bf16_t);
   else if (tx == 1) HNR(bf16_t, float);
   else if (to == 1) HNR(float, bf16_t);
@@ -475,6 +495,74 @@ __global__ __launch_bounds__(256) void moe_hist_kernel(const int* __restrict__ i
   __syncthreads();
   for (int e = threadIdx.x; e < E; e += 256)
     if (h[e]) atomicAdd(hist + e, h[e]);
+}
+
+// one thread per token: scores sigmoid(logit); the experts form `groups` equal groups of neighbours, a group is worth the
+// sum of its two largest scores, only experts of the `keep` best groups compete (ties: the lower group / expert);
+// weights = score / (sum of the chosen + 1e-20) * scale.  groups <= 1: every expert competes
+#define MOE_MAX_GROUPS 64
+__global__ void moe_route_grouped_kernel(const float* __restrict__ logits, int ldl, int T, int E, int top, int groups, int keep,
+                                         float scale, int* __restrict__ ids, float* __restrict__ w) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* l = logits + (size_t)t * ldl;
+  unsigned long long kept = ~0ull;
+  const int per = groups > 1 ? E / groups : E;
+  if (groups > 1) {
+    float worth[MOE_MAX_GROUPS];
+    for (int g = 0; g < groups; ++g) {
+      float b1 = -1.f, b2 = -1.f;                     // (scores lie in (0, 1))
+      for (int e = g * per; e < (g + 1) * per; ++e) {
+        const float sc = sigmoid_f(l[e]);
+        if (sc > b1) { b2 = b1; b1 = sc; } else if (sc > b2) { b2 = sc; }
+      }
+      worth[g] = b1 + (b2 > 0.f ? b2 : 0.f);
+    }
+    kept = 0ull;
+    for (int k = 0; k < keep; ++k) {
+      float best = -1.f;
+      int bg = 0;
+      for (int g = 0; g < groups; ++g)
+        if (!((kept >> g) & 1ull) && worth[g] > best) { best = worth[g]; bg = g; }
+      kept |= 1ull << bg;
+    }
+  }
+  int chosen[MOE_MAX_TOP];
+  float val[MOE_MAX_TOP];
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float best = -1.f;
+    int be = 0;
+    for (int e = 0; e < E; ++e) {
+      if (groups > 1 && !((kept >> (e / per)) & 1ull)) continue;
+      bool used = false;
+      for (int j = 0; j < k; ++j) used |= (chosen[j] == e);
+      if (used) continue;
+      const float sc = sigmoid_f(l[e]);
+      if (sc > best) { best = sc; be = e; }
+    }
+    chosen[k] = be;
+    val[k] = best;
+    sum += best;
+  }
+  const float inv = scale / (sum + 1e-20f);
+  for (int k = 0; k < top; ++k) {
+    ids[(size_t)t * top + k] = chosen[k];
+    w[(size_t)t * top + k] = val[k] * inv;
+  }
+}
+
+extern "C" int fls_seq_moe_route_grouped(const float* logits, int ldl, int T, int E, int top, int groups, int keep, float scale,
+                                         int* ids, float* w, int* hist, fls_stream_t s) {
+  if (T <= 0) return 0;
+  if (top < 1 || top > MOE_MAX_TOP || top > E || E > MOE_MAX_E || groups < 0 || groups > MOE_MAX_GROUPS) return -1;
+  if (groups > 1 && (E % groups || keep < 1 || keep > groups || keep * (E / groups) < top)) return -1;
+  hipLaunchKernelGGL(moe_route_grouped_kernel, dim3((T + 127) / 128), dim3(128), 0, (hipStream_t)s, logits, ldl, T, E, top, groups,
+                     keep, scale, ids, w);
+  SEQ_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_hist_kernel, dim3((T * top + 4095) / 4096), dim3(256), 0, (hipStream_t)s, ids, T * top, E, hist);
+  SEQ_LAUNCH_CHECK();
+  return 0;
 }
 
 extern "C" int fls_seq_moe_route(const float* logits, int ldl, const float* corr, int T, int E, int top, int* ids, float* w,
@@ -576,4 +664,4 @@ extern "C" int fls_seq_moe_combine(float* x, int ldx, const float* y, int ldy, c
   return 0;
 }
 
-extern "C" int fls_seq_version(void) { return 9; }
+extern "C" int fls_seq_version(void) { return 10; }

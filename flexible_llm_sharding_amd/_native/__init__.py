@@ -130,7 +130,7 @@ def _load_kernels(path: str = _KERNELS):
     return lib
 
 
-SEQ_ABI = 9   # csrc/include/fls_seq.h
+SEQ_ABI = 10   # csrc/include/fls_seq.h
 
 
 def _load_seq():
@@ -152,15 +152,15 @@ def _load_seq():
     _bind(lib, "fls_seq_xielu", i, p, i, p, p, i, i, i, i, p)
     _bind(lib, "fls_seq_gate_mul", i, p, i, p, i, i, i, i, i, p)
     _bind(lib, "fls_seq_unary", i, p, i, p, i, i, i, i, i, p)
-    _bind(lib, "fls_seq_head_norm_rope", i, p, i, i, i, i, i, i, p, f, p, i, p, p, p, i, i, i, i, p, i, i, i, p)
+    _bind(lib, "fls_seq_head_norm_rope", i, p, i, i, i, i, i, i, p, f, p, i, p, p, p, i, i, i, i, p, i, i, i, i, f, p)
     _bind(lib, "fls_seq_delta_rule_scan", i, p, i, p, i, p, i, p, i, p, i, p, i, p, p, p, p, i, i, p, p, p, i, i, i, i, f, f, f, f, i, p, p)
     _bind(lib, "fls_seq_softcap", i, p, i, i, i, f, p)
     _bind(lib, "fls_seq_argmax", i, p, i, i, i, p, p)
     _bind(lib, "fls_seq_kv_store", i, p, i, p, f, p, i, p, p, i, p, i, i, i, p)
-    _bind(lib, "fls_seq_attn_paged", i, p, i, i, p, i, p, i, i, p, i, p, p, p, i, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i, i, p,
-          i, f, p, i, p)
-    _bind(lib, "fls_seq_attn_prefill", i, p, i, i, p, i, p, i, p, i, p, i, p, p, p, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i,
-          i, f, p, i, p)
+    _bind(lib, "fls_seq_attn_paged", i, p, i, i, p, i, p, i, i, p, i, i, p, p, p, i, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i, i, p,
+          i, f, p, i, i, p)
+    _bind(lib, "fls_seq_attn_prefill", i, p, i, i, p, i, p, i, p, i, i, p, i, p, p, p, i, i, i, i, i, f, f, p, p, i, i, i, p, f, i,
+          i, f, p, i, i, p)
     _bind(lib, "fls_seq_attn_heads", i, p, i, p, i, p, i, p, i, p, p, p, i, i, i, i, i, i, f, i, i, f, i, i, p, p)
     _bind(lib, "fls_seq_causal_conv", i, p, i, p, p, p, p, i, i, p, p, p, p, i, i, i, i, i, i, i, p)
     _bind(lib, "fls_seq_rglru_scan", i, p, i, p, i, p, p, i, p, p, i, i, p, p, p, i, i, f, p)
@@ -170,6 +170,14 @@ def _load_seq():
     _bind(lib, "fls_seq_moe_scan", i, p, i, p, p, p)
     _bind(lib, "fls_seq_moe_place", i, p, i, i, p, p, p, p)
     _bind(lib, "fls_seq_moe_sum", i, p, i, p, p, p, i, i, i, i, p)
+    _bind(lib, "fls_seq_moe_route_grouped", i, p, i, i, i, i, i, i, f, p, p, p, p)
+    _bind(lib, "fls_seq_embed_pos", i, p, p, i, p, p, p, i, i, i, i, f, i, p)
+    _bind(lib, "fls_seq_streams_norm", i, p, i, p, p, p, p, i, i, i, i, i, f, p)
+    _bind(lib, "fls_seq_streams_update", i, p, i, p, i, p, i, p, f, i, i, i, p, p, p, i, i, f, p)
+    _bind(lib, "fls_seq_scale", i, p, i, i, i, f, p)
+    _bind(lib, "fls_seq_sigmoid_gate", i, p, i, i, p, i, p, i, i, i, i, p)
+    _bind(lib, "fls_seq_diff_combine", i, p, i, p, i, f, i, i, f, p, i, i, i, p)
+    _bind(lib, "fls_seq_hgrn2_scan", i, p, i, p, i, p, i, p, p, p, p, i, p, p, p, i, i, i, i, p)
     return lib
 
 

@@ -55,13 +55,24 @@ class HipSeqOps:
         self._freqs = {}
 
     # ----------------------------------------------------------------- rows
-    def embed_rows(self, ids, table, out=None, scale=1.0):
+    def embed_rows(self, ids, table, out=None, scale=1.0, pos_table=None, tok_pos=None, copies=1):
         T, (V, D) = ids.numel(), table.shape
         if out is None:
-            out = torch.empty(T, D, dtype=torch.float32, device=table.device)
-        if out.dtype != torch.float32 or not out.is_contiguous() or tuple(out.shape) != (T, D):
-            raise TypeError("embed_rows: out must be a contiguous fp32 [T, D] tensor")
+            out = torch.empty(T, D * copies, dtype=torch.float32, device=table.device)
+        if out.dtype != torch.float32 or not out.is_contiguous() or tuple(out.shape) != (T, D * copies):
+            raise TypeError("embed_rows: out must be a contiguous fp32 [T, copies * D] tensor")
         _vec(ids, "ids", T, torch.int32)
+        if pos_table is not None or copies != 1:
+            if pos_table is not None:
+                if pos_table.dtype != table.dtype or pos_table.shape[1] != D or not pos_table.is_contiguous() or not table.is_contiguous():
+                    raise TypeError("embed_rows: pos_table must be laid out like table")
+                _vec(tok_pos, "tok_pos", T, torch.int32)
+            _chk(self.k.fls_seq_embed_pos(ids.data_ptr(), table.data_ptr(), _code(table, "table"),
+                                          pos_table.data_ptr() if pos_table is not None else None,
+                                          tok_pos.data_ptr() if pos_table is not None else None, out.data_ptr(), T, D, V,
+                                          pos_table.shape[0] if pos_table is not None else 0, float(scale), int(copies), _stream()),
+                 "fls_seq_embed_pos")
+            return out
         _chk(self.k.fls_seq_embed(ids.data_ptr(), table.data_ptr(), _code(table, "table"), out.data_ptr(), T, D, V,
                                   float(scale), _stream()), "fls_seq_embed")
         return out
@@ -126,6 +137,123 @@ class HipSeqOps:
                                            alpha.data_ptr(), h.data_ptr(), _CODE[out_dtype], D, T, D, _stream()),
              "fls_seq_add_scaled_dyt")
         return h
+
+    def streams_norm(self, xs, coef, w, eps, out_dtype, streams, row_idx=None):
+        _rows(xs, "xs", torch.float32)
+        D = xs.shape[1] // streams
+        if xs.shape[1] != streams * D:
+            raise ValueError("streams_norm: the row is not streams * D wide")
+        rows = xs.shape[0] if row_idx is None else row_idx.numel()
+        _vec(w, "w", D)
+        if coef is not None and (coef.dtype != torch.float32 or not coef.is_contiguous() or coef.numel() < streams):
+            raise TypeError("streams_norm: coef must be fp32 with at least one entry per stream")
+        if row_idx is not None:
+            _vec(row_idx, "row_idx", rows, torch.int32)
+        y = torch.empty(rows, D, dtype=out_dtype, device=xs.device)
+        _chk(self.k.fls_seq_streams_norm(xs.data_ptr(), xs.stride(0), row_idx.data_ptr() if row_idx is not None else None,
+                                         coef.data_ptr() if coef is not None else None, w.data_ptr(), y.data_ptr(),
+                                         _CODE[out_dtype], D, rows, D, streams, float(eps), _stream()), "fls_seq_streams_norm")
+        return y
+
+    def _streams_update(self, xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype):
+        _rows(xs, "xs", torch.float32)
+        _rows(y, "y", torch.float32)
+        T, D = y.shape
+        if tuple(xs.shape) != (T, streams * D):
+            raise ValueError("streams_update_: xs must be [T, streams * D]")
+        if gate is not None:
+            _rows(gate, "gate", torch.float32)
+            if tuple(gate.shape) != (T, D):
+                raise ValueError("streams_update_: gate is [T, D]")
+        if hc is not None:
+            _vec(hc, "hc", 2 * streams + streams * streams)
+        elif streams != 1:
+            raise ValueError("streams_update_: several streams need their coefficients")
+        h = None
+        if w is not None:
+            _vec(w, "w", D)
+            if coef is not None and (coef.dtype != torch.float32 or not coef.is_contiguous() or coef.numel() < streams):
+                raise TypeError("streams_update_norm_: coef must be fp32 with at least one entry per stream")
+            h = torch.empty(T, D, dtype=out_dtype, device=xs.device)
+        _chk(self.k.fls_seq_streams_update(xs.data_ptr(), xs.stride(0), y.data_ptr(), y.stride(0),
+                                           gate.data_ptr() if gate is not None else None, gate.stride(0) if gate is not None else 0,
+                                           hc.data_ptr() if hc is not None else None, float(mult), T, D, streams,
+                                           coef.data_ptr() if (w is not None and coef is not None) else None,
+                                           w.data_ptr() if w is not None else None, h.data_ptr() if h is not None else None,
+                                           _CODE[out_dtype] if h is not None else 0, D, float(eps), _stream()),
+             "fls_seq_streams_update")
+        return h
+
+    def streams_update_(self, xs, y, gate, hc, mult, streams):
+        self._streams_update(xs, y, gate, hc, mult, streams, None, None, 0.0, torch.float32)
+        return xs
+
+    def streams_update_norm_(self, xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype):
+        return self._streams_update(xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype)
+
+    def scale_(self, z, alpha):
+        _rows(z, "z", torch.float32)
+        _chk(self.k.fls_seq_scale(z.data_ptr(), z.stride(0), z.shape[0], z.shape[1], float(alpha), _stream()), "fls_seq_scale")
+        return z
+
+    def sigmoid_gate(self, o, g, out_dtype):
+        _rows(o, "o")
+        _rows(g, "g", torch.float32)
+        if o.shape != g.shape:
+            raise ValueError("sigmoid_gate: shapes differ")
+        y = torch.empty(o.shape, dtype=out_dtype, device=o.device)
+        _chk(self.k.fls_seq_sigmoid_gate(o.data_ptr(), _code(o, "o"), o.stride(0), g.data_ptr(), g.stride(0), y.data_ptr(),
+                                         _CODE[out_dtype], y.stride(0), o.shape[0], o.shape[1], _stream()), "fls_seq_sigmoid_gate")
+        return y
+
+    def diff_combine(self, a, lam_w, diff, H, dv, eps, out_dtype):
+        _rows(a, "a", torch.float32)
+        if a.shape[1] != 2 * H * dv or lam_w.dim() != 2 or lam_w.shape[0] != 4:
+            raise ValueError("diff_combine: a is [T, 2 H dv], lam_w [4, d]")
+        _vec(lam_w, "lam_w", lam_w.numel())
+        out = torch.empty(a.shape[0], H * dv, dtype=out_dtype, device=a.device)
+        _chk(self.k.fls_seq_diff_combine(a.data_ptr(), a.stride(0), lam_w.data_ptr(), lam_w.shape[1], float(diff), H, dv, float(eps),
+                                         out.data_ptr(), _CODE[out_dtype], out.stride(0), a.shape[0], _stream()), "fls_seq_diff_combine")
+        return out
+
+    def hgrn2_scan(self, q, f, v, fb, lower, norm_w, state, meta, heads, dim, vdim, eps, out_dtype):
+        T = q.shape[0]
+        for nme, t, n in (("q", q, heads * dim), ("f", f, heads * dim), ("v", v, heads * vdim)):
+            _rows(t, nme, torch.float32)
+            if tuple(t.shape) != (T, n):
+                raise ValueError(f"hgrn2_scan: {nme} is {tuple(t.shape)}, not {(T, n)}")
+        _vec(lower, "lower", heads * dim)
+        _vec(norm_w, "norm_w", vdim)
+        if fb is not None:
+            _vec(fb, "fb", heads * dim)
+        if tuple(state.shape[1:]) != (heads, dim, vdim) or not state.is_contiguous() or state.dtype != torch.float32:
+            raise ValueError("hgrn2_scan: state must be fp32 [slots, heads, dim, vdim]")
+        raw = torch.empty(T, heads * vdim, dtype=torch.float32, device=q.device)
+        _chk(self.k.fls_seq_hgrn2_scan(q.data_ptr(), q.stride(0), f.data_ptr(), f.stride(0), v.data_ptr(), v.stride(0),
+                                       fb.data_ptr() if fb is not None else None, lower.data_ptr(), state.data_ptr(),
+                                       raw.data_ptr(), raw.stride(0), meta["cu"].data_ptr(), meta["pos0"].data_ptr(),
+                                       meta["slot"].data_ptr(), meta["n_seqs"], heads, dim, vdim, _stream()), "fls_seq_hgrn2_scan")
+        out = torch.empty(T, heads * vdim, dtype=out_dtype, device=q.device)
+        # every head's output over its own root mean square, times the weight the heads share
+        return self.head_norm_rope(raw, heads, vdim, 0, vdim, out, 0, vdim, meta, w=norm_w, eps=eps)
+
+    def moe_route_grouped(self, logits, top, groups, keep, scale):
+        _rows(logits, "logits", torch.float32)
+        T, E = logits.shape
+        dev = logits.device
+        ids = torch.empty(T, top, dtype=torch.int32, device=dev)
+        w = torch.empty(T, top, dtype=torch.float32, device=dev)
+        ints = torch.zeros(3 * E + 1, dtype=torch.int32, device=dev)          # hist | cursor | offs
+        hist, cursor, offs = ints[:E], ints[E:2 * E], ints[2 * E:]
+        dest = torch.empty(T, top, dtype=torch.int32, device=dev)
+        rows = torch.empty(T * top, dtype=torch.int32, device=dev)
+        s = _stream()
+        _chk(self.k.fls_seq_moe_route_grouped(logits.data_ptr(), logits.stride(0), T, E, top, int(groups or 0), int(keep or 0),
+                                              float(scale), ids.data_ptr(), w.data_ptr(), hist.data_ptr(), s), "fls_seq_moe_route_grouped")
+        _chk(self.k.fls_seq_moe_scan(hist.data_ptr(), E, offs.data_ptr(), cursor.data_ptr(), s), "fls_seq_moe_scan")
+        _chk(self.k.fls_seq_moe_place(ids.data_ptr(), T * top, top, cursor.data_ptr(), dest.data_ptr(), rows.data_ptr(), s),
+             "fls_seq_moe_place")
+        return SeqRoute(ids, w, offs, rows, dest, top)
 
     def qkv_conv_rope_store(self, z, w, state, meta, H, G, d, dv, q_out, kc, vc, eps=0.0, rot=None):
         _rows(z, "z", torch.float32)
@@ -236,11 +364,11 @@ class HipSeqOps:
 
     def unary(self, z, kind, out_dtype):
         _rows(z, "z", torch.float32)
-        if kind != "tanh":
+        if kind not in ("tanh", "gelu"):
             raise ValueError(kind)
         y = torch.empty(z.shape, dtype=out_dtype, device=z.device)
         _chk(self.k.fls_seq_unary(z.data_ptr(), z.stride(0), y.data_ptr(), _CODE[out_dtype], z.shape[1], z.shape[0],
-                                  z.shape[1], 0, _stream()), "fls_seq_unary")
+                                  z.shape[1], 1 if kind == "gelu" else 0, _stream()), "fls_seq_unary")
         return y
 
     def unfolded_attention_ok(self, dk, dv, cdt):
@@ -267,7 +395,7 @@ class HipSeqOps:
         return self._freqs[key]
 
     def head_norm_rope(self, x, heads, n, x_col, x_hs, out, out_col, out_hs, meta, w=None, eps=0.0, rot=None,
-                       row_map=None, raw=None, unit_after=False):
+                       row_map=None, raw=None, unit_after=False, half=False):
         _rows(x, "x")
         _rows(out, "out")
         T = x.shape[0]
@@ -282,17 +410,21 @@ class HipSeqOps:
             raise ValueError("head_norm_rope: raw must be laid out like out")
         if w is not None:
             _vec(w, "w", n)
-        dims, freqs = 0, None
+        dims, freqs, amp = 0, None, 1.0
         if rot is not None and rot[0] > 0:
+            from .torch_seq import TorchSeqOps
             dims = int(rot[0])
-            freqs = self.rope_freqs(dims, rot[1], x.device, rot[2] if len(rot) > 2 else None)
+            sc = rot[2] if len(rot) > 2 else None
+            freqs = self.rope_freqs(dims, rot[1], x.device, sc)
+            amp = TorchSeqOps.rope_amp(sc)
         _chk(self.k.fls_seq_head_norm_rope(x.data_ptr(), _code(x, "x"), x.stride(0), x_col, x_hs, heads, n,
                                            w.data_ptr() if w is not None else None, float(eps),
                                            freqs.data_ptr() if freqs is not None else None, dims, meta["tok_pos"].data_ptr(),
                                            row_map.data_ptr() if row_map is not None else None, out.data_ptr(),
                                            _code(out, "out"), out.stride(0), out_col, out_hs,
                                            raw.data_ptr() if raw is not None else None,
-                                           raw.stride(0) if raw is not None else 0, T, 1 if unit_after else 0, _stream()),
+                                           raw.stride(0) if raw is not None else 0, T, 1 if unit_after else 0,
+                                           1 if half else 0, float(amp), _stream()),
              "fls_seq_head_norm_rope")
         return out
 
@@ -333,14 +465,17 @@ class HipSeqOps:
                                      kcols, vcols, _stream()), "fls_seq_kv_store")
 
     def attn_paged(self, q, kcache, vcache, meta, H, G, d, dv, scale, softcap, r1, r2, chunk, page_size, out_dtype,
-                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None, sink=None, head_gate=None):
+                   window=0, keep_first=0, gate_bias=None, out_scale=1.0, out=None, sink=None, head_gate=None, v_heads=None):
         _rows(q, "q")
         T = q.shape[0]
         if kcache.dtype != out_dtype or vcache.dtype != out_dtype or q.shape[1] != H * d \
                 or (q.dtype != out_dtype and q.dtype != torch.float32):
-            raise TypeError("attn_paged: the pools and the output share one element type; q is [T, H d] of it or fp32")
+            raise TypeError("attn_paged: the pools share one element type (out_dtype); q is [T, H d] of it or fp32")
         ldk, ldv = kcache.shape[-1], vcache.shape[-1]
-        if ldk < G * d or ldv < G * dv or kcache.shape[1] != page_size or not kcache.is_contiguous() \
+        Gv = int(v_heads or G)
+        if G % Gv:
+            raise ValueError("attn_paged: v_heads must divide the key heads")
+        if ldk < G * d or ldv < Gv * dv or kcache.shape[1] != page_size or not kcache.is_contiguous() \
                 or not vcache.is_contiguous():
             raise ValueError("attn_paged: pools do not fit the head sizes")
         table = meta["page_table"]
@@ -351,9 +486,10 @@ class HipSeqOps:
             raise ValueError("attn_paged: r1 and r2 come together")
         if out is None:
             out = torch.empty(T, H * dv, dtype=out_dtype, device=q.device)
-        elif out.dtype != out_dtype or tuple(out.shape) != (T, H * dv):
+        elif (out.dtype != out_dtype and out.dtype != torch.float32) or tuple(out.shape) != (T, H * dv):
             raise TypeError("attn_paged: out does not fit")
         _rows(out, "out")
+        to = _code(out, "out")
         if head_gate is not None:
             _rows(head_gate, "head_gate", torch.float32)
             if tuple(head_gate.shape) != (T, H):
@@ -366,13 +502,13 @@ class HipSeqOps:
         if tiles is not None and kcache.dtype == torch.bfloat16 and d in (64, 128) and dv in (64, 128):
             # a step with many rows per request: the matrix-core kernel over row tiles
             rc = self.k.fls_seq_attn_prefill(q.data_ptr(), q.stride(0), _code(q, "q"), kcache.data_ptr(), ldk, vcache.data_ptr(),
-                                             ldv, out.data_ptr(), out.stride(0), tiles.data_ptr(), tiles.shape[0],
+                                             ldv, out.data_ptr(), to, out.stride(0), tiles.data_ptr(), tiles.shape[0],
                                              meta["tok_seq"].data_ptr(), meta["tok_pos"].data_ptr(), table.data_ptr(),
                                              table.stride(0), H, G, d, dv, float(scale), float(softcap),
                                              r1.data_ptr() if r1 is not None else None,
                                              r2.data_ptr() if r2 is not None else None, int(chunk), int(window),
                                              int(keep_first), gate_bias.data_ptr() if gate_bias is not None else None,
-                                             float(out_scale), int(page_size), *extra, _stream())
+                                             float(out_scale), int(page_size), *extra, Gv, _stream())
             if rc == 0:
                 return out
             if rc != -2:
@@ -383,7 +519,8 @@ class HipSeqOps:
         if window > 0:
             bound = min(bound, int(window) + int(keep_first))
         if tiles is None and q.dtype == torch.float32 and kcache.dtype == torch.bfloat16 and gate_bias is None and r1 is None \
-                and sink is None and head_gate is None and softcap == 0 and chunk == 0 and H // G <= 32 and (d, dv) in self.HEAD_TILE_SHAPES:
+                and sink is None and head_gate is None and softcap == 0 and chunk == 0 and H // G <= 32 and Gv == G and to == 1 \
+                and (d, dv) in self.HEAD_TILE_SHAPES:
             # few rows whose heads share long key / value rows (decoding over cached latent rows): the heads of a
             # token as the columns of one matrix-core tile, every key tile staged once for all of them
             ns = max(1, min(16, 256 // max(1, T * G), bound // 32))
@@ -402,12 +539,12 @@ class HipSeqOps:
         nsplit = max(1, min(8, 512 // max(1, T * H), bound // 256))
         part = torch.empty(T * H * nsplit * (dv + 4), dtype=torch.float32, device=q.device) if nsplit > 1 else None
         _chk(self.k.fls_seq_attn_paged(q.data_ptr(), q.stride(0), _code(q, "q"), kcache.data_ptr(), ldk, vcache.data_ptr(), ldv,
-                                       _code(kcache, "kcache"), out.data_ptr(), out.stride(0), meta["tok_seq"].data_ptr(),
+                                       _code(kcache, "kcache"), out.data_ptr(), to, out.stride(0), meta["tok_seq"].data_ptr(),
                                        meta["tok_pos"].data_ptr(), table.data_ptr(), table.stride(0), T, H, G, d, dv,
                                        float(scale), float(softcap), r1.data_ptr() if r1 is not None else None,
                                        r2.data_ptr() if r2 is not None else None, int(chunk), int(window), int(keep_first),
                                        gate_bias.data_ptr() if gate_bias is not None else None, float(out_scale),
-                                       int(page_size), nsplit, part.data_ptr() if part is not None else None, *extra,
+                                       int(page_size), nsplit, part.data_ptr() if part is not None else None, *extra, Gv,
                                        _stream()), "fls_seq_attn_paged")
         return out
 

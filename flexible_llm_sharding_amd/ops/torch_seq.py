@@ -79,7 +79,7 @@ class TorchSeqOps:
         if row_idx is not None:
             xs = xs.index_select(0, row_idx.long())
         T = xs.shape[0]
-        x3 = xs.float().reshape(T, streams, -1)
+        x3 = xs.float().reshape(T, streams, xs.shape[1] // streams)
         u = x3.sum(1) if coef is None else torch.einsum("s,tsd->td", coef.float()[:streams], x3)
         return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
 
@@ -88,7 +88,7 @@ class TorchSeqOps:
         ``hc`` = [in (streams) | out (streams) | mix (streams x streams, [from, to])] fp32, None: one stream
         that keeps itself (a plain residual sum); ``gate`` [T, D] fp32 logits or None."""
         T = xs.shape[0]
-        x3 = xs.reshape(T, streams, -1)
+        x3 = xs.reshape(T, streams, xs.shape[1] // streams)
         yy = y.float()
         if gate is not None:
             yy = yy * torch.sigmoid(gate.float())

@@ -1,0 +1,327 @@
+"""Lopilix through the framework (config registry, weight images, sequence state cache, step
+scheduler, kernels) against the plain float64 oracle in ``lopilix_oracle.py``.
+
+Every test runs on the CPU backend (plain PyTorch ops) and, marked ``gpu``, on the HIP kernels.  The
+models are tiny and random; fp32 matrix products make the comparison sharp (a key one place off, a
+lost recurrent state, a pass of a looped layer that reads another pass's keys, a wrong page or a
+forgotten stream coefficient shows as an error thousands of times the tolerance), and some tests run
+the bf16 mode.  Where random weights would hide a fault, the weights are set so that one key dominates."""
+import json
+import math
+import os
+import pickle
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import lopilix_oracle as oracle
+import lopilix_util as lu
+from conftest import gpu_available
+from flexible_llm_sharding_amd.runtime.batch import StepEntry
+from flexible_llm_sharding_amd.serve import generate, load_runner
+
+DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
+TOL = 2e-4          # fp32 products against float64, relative to a logit row's spread
+F = torch.float64
+
+
+@pytest.fixture(autouse=True)
+def _need_gpu(request):
+    params = getattr(getattr(request.node, "callspec", None), "params", {})
+    if "cuda" in str(params.get("device", "")) and not gpu_available():
+        pytest.skip("no GPU")
+
+
+def build(tmp_path, layers, seed=0, dtype=torch.float32, device="cpu", **kw):
+    cfg = lu.config(layers, **{k: v for k, v in kw.items() if k in ("width", "vocab", "eps", "mult", "streams", "logit_scale", "loop",
+                                                                     "max_positions")})
+    sd = lu.random_weights(cfg, seed, **({"std": kw["std"]} if "std" in kw else {}))
+    path = lu.write_model(str(tmp_path / f"m{seed}"), cfg, sd)
+    runner = load_runner(path, dtype, device, max_tokens=kw.get("max_tokens", 64), max_seqs=kw.get("max_seqs", 2),
+                         layer_num_per_shard=kw.get("lnps"), token_budget=kw.get("token_budget", 16384),
+                         resident=kw.get("resident", True))
+    return cfg, sd, runner, path
+
+
+def run_cut(runner, rid, toks, cuts, end=True):
+    """Feed ``toks`` in portions of the sizes ``cuts`` (the rest one by one) -> logits of every position."""
+    out, at = [], 0
+    sizes = list(cuts) + [1] * (len(toks) - sum(cuts))
+    for n in sizes:
+        last = at + n == len(toks)
+        r = runner.step([StepEntry(rid, toks[at:at + n], range(n))], [rid] if (last and end) else [])
+        out.append(r[0][0])
+        at += n
+    return np.concatenate(out, 0)
+
+
+# differential attention + dense, HGRN2 + experts, latent attention + experts without groups, HGRN2 without a
+# feed-forward, a multi-head differential attention whose whole head is rotated; layers 1 .. 3 run twice
+STACK = [(lu.attn(), lu.dense()),
+         (lu.hgrn(), lu.moe()),
+         (lu.latent(), lu.moe(experts=5, top=3, ff=9, groups=None, scale=0.8)),
+         (lu.hgrn(heads=2, dim=20, vdim=6), None),
+         (lu.attn(heads=3, kv_heads=3, dim=8, vdim=5, rot_dims=8, base=1000.0, scale=0.7, diff=0.6), lu.moe(experts=4, top=4, ff=10, groups=(2, 2)))]
+LOOP = (1, 4, 2)
+
+
+# ------------------------------------------------------------------ each mechanism alone
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,layers,kw", [
+    ("differential-attention", [(lu.attn(scale=1.5), None)], {}),
+    ("differential-attention-one-head-no-rotation", [(lu.attn(heads=1, kv_heads=1, dim=4, vdim=3, rot_dims=0), None)], {}),
+    ("differential-attention-multi-head-full-rotation", [(lu.attn(heads=3, kv_heads=3, dim=8, vdim=8, rot_dims=8), None)], {}),
+    ("hgrn2", [(lu.hgrn(), None)], {}),
+    ("hgrn2-one-head-wide-state", [(lu.hgrn(heads=1, dim=37, vdim=70), None)], {}),
+    ("hgrn2-narrow", [(lu.hgrn(heads=5, dim=1, vdim=1), None)], {}),
+    ("latent-attention", [(lu.latent(), None)], {}),
+    ("latent-attention-unscaled-rotation", [(lu.latent(scaling=None, heads=1, kv_rank=3, vdim=12), None)], {}),
+    ("latent-attention-every-pair-slowed", [(lu.latent(scaling={"factor": 2.0, "original": 8, "fast": 64.0, "slow": 32.0}), None)], {}),
+    ("dense-feed-forward", [(lu.hgrn(), lu.dense(ff=33))], {}),
+    ("experts-grouped", [(lu.hgrn(), lu.moe(experts=12, top=3, groups=(4, 2)))], {}),
+    ("experts-groups-of-one", [(lu.hgrn(), lu.moe(experts=5, top=2, groups=(5, 3)))], {}),
+    ("experts-all-groups-kept-all-chosen", [(lu.hgrn(), lu.moe(experts=4, top=4, groups=(2, 2), scale=1.0))], {}),
+    ("experts-top-1-no-groups", [(lu.hgrn(), lu.moe(experts=7, top=1, groups=None))], {}),
+    ("one-stream", [(lu.attn(), lu.dense()), (lu.hgrn(), lu.moe())], {"streams": 1}),
+    ("five-streams", [(lu.attn(), lu.dense()), (lu.latent(), None)], {"streams": 5}),
+    ("unit-multipliers", [(lu.attn(), lu.moe())], {"mult": 1.0, "logit_scale": 1.0}),
+    ("loop-of-one-layer-three-times", [(lu.attn(), None), (lu.hgrn(), lu.dense()), (lu.latent(), None)], {"loop": (1, 2, 3)}),
+    ("loop-once", [(lu.attn(), None), (lu.hgrn(), lu.dense())], {"loop": (0, 2, 1)}),
+    ("width-not-a-multiple-of-four", [(lu.attn(), lu.moe()), (lu.latent(), lu.dense())], {"width": 34}),
+])
+def test_mechanism_alone(tmp_path, device, name, layers, kw):
+    cfg, sd, runner, _ = build(tmp_path, layers, seed=3, device=device, **kw)
+    toks = lu.tokens(45, cfg["vocab"], 1)
+    want = lu.oracle_logits(cfg, sd, toks)
+    assert lu.rel_err(run_cut(runner, "a", toks, [len(toks)]), want) < TOL
+    assert lu.rel_err(run_cut(runner, "b", toks, [30, 2]), want) < TOL
+    runner.close()
+
+
+def test_oracle_parts_agree_with_their_definitions():
+    """The oracle's own pieces on hand-made inputs: both pair layouts of the rotation, the rescaled
+    frequencies and their amplitude, the recurrence by hand, routing among groups, lambda, the layer order."""
+    x = torch.tensor([[[0.0, 0.0, 5.0, 6.0, 7.0]], [[1.0, 0.0, 0.0, 2.0, 7.0]]], dtype=F)
+    r = oracle.rotate(x, {"dims": 2, "base": 100.0}, "pairs")
+    assert torch.allclose(r[1, 0], torch.tensor([math.cos(1.0), math.sin(1.0), 0.0, 2.0, 7.0], dtype=F))
+    r = oracle.rotate(x, {"dims": 4, "base": 100.0}, "half")           # pairs (0, 2) and (1, 3); f = 1, 0.1
+    assert torch.allclose(r[1, 0], torch.tensor([math.cos(1.0), -2 * math.sin(0.1), math.sin(1.0), 2 * math.cos(0.1), 7.0], dtype=F))
+    assert torch.equal(r[0], x[0])
+    rot = {"dims": 16, "base": 100.0, "scaling": {"factor": 8.0, "original": 64, "fast": 4.0, "slow": 1.0}}
+    f, amp = oracle.rot_freqs(rot)
+    f0, one = oracle.rot_freqs({"dims": 16, "base": 100.0})
+    ratio = [a / b for a, b in zip(f, f0)]
+    assert one == 1.0 and abs(amp - (0.1 * math.log(8.0) + 1.0)) < 1e-15
+    # entry numbers where a pair turns 4 times and once over 64 positions: 16 ln(64 / (2 pi t)) / (2 ln 100)
+    lo, hi = math.floor(16 * math.log(64 / (8 * math.pi)) / (2 * math.log(100))), math.ceil(16 * math.log(64 / (2 * math.pi)) / (2 * math.log(100)))
+    assert (lo, hi) == (1, 5)
+    assert ratio[0] == 1.0 and ratio[1] == 1.0 and abs(ratio[3] - (1 - 0.5 + 0.5 / 8)) < 1e-12 and all(abs(q - 1 / 8) < 1e-12 for q in ratio[5:])
+    # the recurrence with one head, one state row and gate 1/2: S = S / 2 + v / 2
+    sd = {"q": torch.tensor([[100.0]], dtype=F), "f": torch.zeros(1, 1, dtype=F), "f.b": torch.zeros(1, dtype=F), "lower": torch.zeros(1, dtype=F),
+          "v": torch.tensor([[1.0], [0.0]], dtype=F), "norm": torch.ones(2, dtype=F), "o": torch.eye(2, dtype=F)}
+    h = torch.tensor([[1.0], [1.0], [1.0]], dtype=F)
+    S = torch.zeros(2, dtype=F)
+    rows = []
+    for t in range(3):
+        S = 0.5 * S + 0.5 * torch.tensor([1.0, 0.0], dtype=F)
+        rows.append(oracle.rms(S * 100.0, 1e-6))
+    assert torch.allclose(oracle.hgrn2(sd, "", {"heads": 1, "dim": 1, "vdim": 2}, h, 1e-6), torch.stack(rows), atol=1e-9)
+    # a lower bound of 1 never forgets and never writes
+    sd["lower"] = torch.ones(1, dtype=F)
+    assert oracle.hgrn2(sd, "", {"heads": 1, "dim": 1, "vdim": 2}, h, 1e-6).abs().max() == 0.0
+    # groups (0,1) (2,3) (4,5): worth 0.9+0.1, 0.6+0.6, 0.7+0.2 -> groups 1 and 0 compete, expert 4 does not
+    logit = lambda p: math.log(p / (1 - p))
+    z = torch.tensor([logit(p) for p in (0.9, 0.1, 0.6, 0.6, 0.7, 0.2)], dtype=F)
+    got = oracle.route(z, {"experts": 6, "top": 3, "scale": 2.0, "groups": {"count": 3, "keep": 2}})
+    assert [e for e, _ in got] == [0, 2, 3] and np.allclose([w for _, w in got], [2 * 0.9 / 2.1, 2 * 0.6 / 2.1, 2 * 0.6 / 2.1])
+    got = oracle.route(z, {"experts": 6, "top": 3, "scale": 1.0})
+    assert [e for e, _ in got] == [0, 4, 2]
+    lam = oracle.diff_lambda({"lq1": torch.tensor([1.0, 2.0], dtype=F), "lk1": torch.tensor([0.5, 0.25], dtype=F),
+                              "lq2": torch.zeros(2, dtype=F), "lk2": torch.ones(2, dtype=F)}, "", 0.2)
+    assert abs(lam - (math.e - 1.0 + 0.2)) < 1e-12
+    assert oracle.layer_order({"layers": [0] * 5, "loop": {"start": 1, "stop": 3, "times": 3}}) == [0, 1, 2, 1, 2, 1, 2, 3, 4]
+    assert oracle.layer_order({"layers": [0] * 2}) == [0, 1]
+
+
+# ----------------------------------------------- prompts, portions, decoding, first tokens
+@pytest.mark.parametrize("device", DEVICES)
+def test_prefill_portions_and_decode(tmp_path, device):
+    """The same sequence whole, token by token, and in portions of 2, 3, 7, 16 and 17 tokens: keys, latent
+    rows and recurrent states of both passes of the looped layers all cross the cuts."""
+    cfg, sd, runner, _ = build(tmp_path, STACK, seed=5, device=device, loop=LOOP)
+    toks = lu.tokens(50, cfg["vocab"], 2)
+    want = lu.oracle_logits(cfg, sd, toks)
+    for cuts in ([50], [], [2, 2, 3, 7, 16, 17], [17, 16, 2], [1, 2, 40]):
+        assert lu.rel_err(run_cut(runner, "r", toks, cuts), want) < TOL, cuts
+    runner.close()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_residual_streams_after_every_layer_run(tmp_path, device):
+    """What leaves every layer run (a looped layer counts each time) against the oracle's summed streams,
+    through the layer functions on the runner's own weights and cache."""
+    cfg, sd, runner, _ = build(tmp_path, STACK, seed=4, device=device, loop=LOOP)
+    toks = lu.tokens(21, cfg["vocab"], 8)
+    trace = []
+    lu.oracle_logits(cfg, sd, toks, trace)
+    from flexible_llm_sharding_amd.runtime.batch import pack_step
+    batch = pack_step([StepEntry("t", toks, [len(toks) - 1])], runner.seq_cache)
+    meta = batch.device_tensors(runner.dev)
+    W = {}
+    for k in range(len(runner.my_shards)):
+        W.update(runner.prefetcher.acquire(k))
+    state, n = None, 0
+    for name in runner.names:
+        state = runner.family.run_layer(runner.ctx, name, W[name], state, batch, meta)
+        if name[0] == "l":
+            got = state.float().reshape(len(toks), cfg["streams"], cfg["width"]).sum(1).cpu().double()
+            assert (got - trace[n]).abs().max() < 1e-4 * trace[n].abs().max(), name
+            n += 1
+    assert n == len(trace) == 8
+    runner.seq_cache.release("t")
+    runner.close()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decoding_over_pages(tmp_path, device):
+    """A short prompt, then 120 decoded tokens: pages of 16 fill one after the other, the recurrent states
+    are carried 120 times, and nothing is ever given back while the request lives (every key stays visible)."""
+    cfg, sd, runner, _ = build(tmp_path, STACK, seed=6, device=device, loop=LOOP)
+    toks = lu.tokens(125, cfg["vocab"], 7)
+    got = run_cut(runner, "r", toks, [5], end=False)
+    assert lu.rel_err(got, lu.oracle_logits(cfg, sd, toks)) < TOL
+    cache = runner.seq_cache
+    assert cache.pages_trimmed == 0 and all(p >= 0 for p in cache.requests["r"].pages) and len(cache.requests["r"].pages) == 8
+    cache.release("r")
+    runner.close()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_first_tokens(tmp_path, device):
+    """Sequences of one, two and three tokens, whole and decoded."""
+    cfg, sd, runner, _ = build(tmp_path, STACK, seed=8, device=device, loop=LOOP)
+    for n in (1, 2, 3):
+        toks = lu.tokens(n, cfg["vocab"], 20 + n)
+        want = lu.oracle_logits(cfg, sd, toks)
+        assert lu.rel_err(run_cut(runner, "w", toks, [n]), want) < TOL
+        assert lu.rel_err(run_cut(runner, "d", toks, []), want) < TOL
+    runner.close()
+
+
+# ------------------------------------------------------------ batches, pages and slots
+@pytest.mark.parametrize("device", DEVICES)
+def test_unequal_batch_equals_each_alone(tmp_path, device):
+    """Requests of 1, 9, 33 and 50 tokens in one step, then decoded together while the short ones
+    finish first; also cut into two micro-batches by a small token budget."""
+    for budget in (16384, 40):
+        cfg, sd, runner, _ = build(tmp_path, STACK, seed=9, device=device, token_budget=budget, loop=LOOP)
+        lens, extra = [1, 9, 33, 50], [3, 12, 0, 6]
+        seqs = [lu.tokens(n + e, cfg["vocab"], 30 + i) for i, (n, e) in enumerate(zip(lens, extra))]
+        want = [lu.oracle_logits(cfg, sd, s) for s in seqs]
+        got = [[] for _ in seqs]
+        live = list(range(4))
+        res = runner.step([StepEntry(i, seqs[i][:lens[i]], range(lens[i])) for i in live], [i for i in live if extra[i] == 0])
+        for i, r in zip(live, res):
+            got[i].append(r[0])
+        for t in range(max(extra)):
+            live = [i for i in range(4) if extra[i] > t]
+            res = runner.step([StepEntry(i, [seqs[i][lens[i] + t]], [0]) for i in live], [i for i in live if extra[i] == t + 1])
+            for i, r in zip(live, res):
+                got[i].append(r[0])
+        for i in range(4):
+            assert lu.rel_err(np.concatenate(got[i], 0), want[i]) < TOL, (budget, i)
+        assert not runner.seq_cache.requests
+        runner.close()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_pages_and_slots_used_again(tmp_path, device):
+    """Requests come and go through pools of two slots and a few pages: whoever inherits a page or a
+    slot (with the last owner's keys, latent rows and recurrent states still in it) computes what it
+    computes alone, and pools that run out grow without disturbing the live request."""
+    cfg, sd, runner, _ = build(tmp_path, STACK, seed=11, device=device, max_tokens=40, max_seqs=2, loop=LOOP)
+    cache = runner.seq_cache
+    a, b, c = (lu.tokens(n, cfg["vocab"], 40 + n) for n in (37, 22, 41))
+    wa, wb, wc = (lu.oracle_logits(cfg, sd, s) for s in (a, b, c))
+    assert lu.rel_err(run_cut(runner, "a", a, [30]), wa) < TOL
+    ga = run_cut(runner, "a2", a, [10, 2], end=False)                       # stays alive
+    gb = run_cut(runner, "b", b, [22])                                      # inherits a's first slot
+    assert cache.slots_reused > 0 and cache.pages_reused > 0
+    gc = run_cut(runner, "c", c, [3, 30])
+    n0 = cache.n_slots
+    others = [run_cut(runner, f"x{i}", b, [5], end=False) for i in range(3)]    # more requests than slots
+    assert cache.n_slots > n0
+    tail = runner.step([StepEntry("a2", [a[0]], [0])], ["a2"])[0][0]         # a2's state survived the growth
+    assert lu.rel_err(tail, lu.oracle_logits(cfg, sd, a + [a[0]])[-1:]) < TOL
+    for g, w in ((ga, wa), (gb, wb), (gc, wc)) + tuple((o, wb) for o in others):
+        assert lu.rel_err(g, w) < TOL
+    runner.close()
+
+
+# ----------------------------------------------------- shards, bf16, generation
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("lnps", [1, 3])
+def test_few_layers_per_shard_stream_weights(tmp_path, device, lnps):
+    """Weights streamed shard by shard: the passes of a looped layer land in different shards (its image is
+    loaded again) or in one (loaded once, shared)."""
+    cfg = lu.config(STACK, loop=LOOP)
+    sd = lu.random_weights(cfg, 13)
+    path = lu.write_model(str(tmp_path / "s"), cfg, sd)
+    runner = load_runner(path, torch.float32, device, max_tokens=64, layer_num_per_shard=lnps, resident=False)
+    toks = lu.tokens(40, cfg["vocab"], 3)
+    assert lu.rel_err(run_cut(runner, "r", toks, [20, 2]), lu.oracle_logits(cfg, sd, toks)) < TOL
+    runner.close()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_bf16_products_stay_close(tmp_path, device):
+    cfg, sd, runner, _ = build(tmp_path, STACK, seed=14, device=device, dtype=torch.bfloat16, loop=LOOP)
+    toks = lu.tokens(40, cfg["vocab"], 4)
+    want = lu.oracle_logits(cfg, sd, toks)
+    whole, cut = run_cut(runner, "a", toks, [40]), run_cut(runner, "b", toks, [9, 2])
+    assert lu.rel_err(whole, want) < 0.15 and lu.rel_err(cut, want) < 0.15      # (the worst row)
+    assert lu.rel_err(cut, whole) < 0.12
+    runner.close()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_head_sizes_of_the_matrix_core_kernels(tmp_path, device):
+    """bf16 with head sizes that the matrix-core prompt attention serves on the GPU (differential attention
+    with keys of 64 and values of 128; latent attention with 64 + 64 wide keys made per head from the step's
+    rows, and a latent of 128 + 64 that the heads-as-columns decode kernel reads): a prompt of several row
+    tiles, a portion that continues it, then decoding.  Whole-prompt and decoded logits both stay within
+    bf16 rounding of the oracle, and of each other."""
+    layers = [(lu.attn(heads=4, kv_heads=2, dim=64, vdim=128, rot_dims=32, base=1e4, scale=0.12), lu.moe()),
+              (lu.latent(heads=4, dim=64, rot_dim=64, vdim=128, kv_rank=128, base=1e4, scale=0.09), None),
+              (lu.attn(heads=2, kv_heads=1, dim=128, vdim=64, rot_dims=128, base=1e4, scale=0.09), lu.dense())]
+    cfg, sd, runner, _ = build(tmp_path, layers, seed=23, device=device, dtype=torch.bfloat16, max_tokens=512, std=0.2)
+    toks = lu.tokens(230, cfg["vocab"], 6)
+    want = lu.oracle_logits(cfg, sd, toks)
+    whole = run_cut(runner, "a", toks, [230])
+    cut = run_cut(runner, "b", toks, [150, 40])
+    # (the difference of two attention maps, divided by its own root mean square, amplifies the rounding of both)
+    assert lu.rel_err(whole, want) < 0.16 and lu.rel_err(cut, want) < 0.16
+    assert lu.rel_err(cut, whole) < 0.12
+    runner.close()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_the_scheduler(tmp_path, device):
+    """serve.generate: prompts of unequal length, 12 new tokens each; the tokens are the oracle's
+    greedy continuation (recomputed from scratch at every step)."""
+    cfg, sd, runner, _ = build(tmp_path, STACK, seed=15, device=device, loop=LOOP)
+    prompts = [lu.tokens(n, cfg["vocab"], 50 + n) for n in (3, 17, 26)]
+    got = generate(runner, prompts, 12)
+    for p, g in zip(prompts, got):
+        seq = list(p)
+        for t in g:
+            z = lu.oracle_logits(cfg, sd, seq)[-1]
+            top2 = np.sort(z)[-2:]
+            if top2[1] - top2[0] > 1e-3:              # (a tie within rounding may go either way)
+                assert t == int(z.argmax())
+            seq.append(t)
+    assert not runner.seq_cache.requests
+    runner.close()
