@@ -388,7 +388,7 @@ class HipSeqOps:
         return out
 
     def rope_freqs(self, dims, base, device, scaling=None):
-        key = (int(dims), float(base), str(device), None if scaling is None else tuple(float(v) for v in scaling))
+        key = (int(dims), float(base), str(device), None if scaling is None else tuple(scaling))
         if key not in self._freqs:
             from .torch_seq import TorchSeqOps
             self._freqs[key] = TorchSeqOps.rope_freqs(int(dims), float(base), device, scaling)
