@@ -325,3 +325,199 @@ def test_greedy_generation_through_the_scheduler(tmp_path, device):
             seq.append(t)
     assert not runner.seq_cache.requests
     runner.close()
+
+
+# ------------------------------------------- one token that stands out, far back and at page borders
+def _marked_model(tmp_path, kind):
+    """One layer whose weights make one marked token decide every later row.  Channel 0 of the embedding is
+    the same for every token, channel 1 is zero except for the marked token, where it is large; positions
+    add next to nothing.  ``attention``: every query of map 1 points along u, every key along -u, the marked
+    token's along +u, so after the per-head norms its score is +scale * dim against -scale * dim for all
+    others, however many hundreds there are.  ``latent``: the latent's first entry carries that sign, W_uk
+    turns it into +-u, the unrotated query is u.  ``hgrn2``: lower bounds next to 1 keep what the marked
+    token wrote (a large value) for hundreds of steps."""
+    D, vocab, mark, d = 24, 40, 7, 8
+    u = torch.tensor([0.0, 0.0, 1.0, -1.0, 1.0, 1.0, -1.0, 1.0])            # (entries 0, 1 are a rotated pair: left out)
+    mixer = {"attention": lu.attn(heads=2, kv_heads=1, dim=d, vdim=6, rot_dims=2, base=1e6, scale=1.6, diff=0.35),
+             "latent": lu.latent(heads=2, dim=d, rot_dim=4, vdim=6, kv_rank=5, base=1e6, scaling=None, scale=0.4),
+             "hgrn2": lu.hgrn(heads=2, dim=4, vdim=6)}[kind]
+    cfg = lu.config([(mixer, None)], width=D, vocab=vocab, mult=1.0, streams=2, logit_scale=1.0, max_positions=320)
+    sd = {k: v.float() for k, v in lu.random_weights(cfg, 12, std=0.05).items()}
+    sd["embed"] *= 0.05
+    sd["pos"] *= 0.02
+    sd["embed"][:, 0] = 4.0
+    sd["embed"][:, 1] = 0.0
+    sd["embed"][mark, 1] = 12.0
+    sd["l0.norm1"][:] = 1.0
+    x = "l0.mix."
+    if kind == "attention":
+        sd[x + "q.norm"][:] = 1.0
+        sd[x + "k.norm"][:] = 1.0
+        for hh in range(2):
+            sd[x + "q"][hh * 2 * d:hh * 2 * d + d, 0] = u                   # map 1 of head hh
+        sd[x + "k"][:d, 0] = -u
+        sd[x + "k"][:d, 1] = u
+        sd[x + "v"][:, 1] = 3.0
+    elif kind == "latent":
+        sd[x + "dkv.norm"][:] = 1.0
+        sd[x + "dkv"][0, 0], sd[x + "dkv"][0, 1] = -1.0, 1.0
+        for hh in range(2):
+            sd[x + "q"][hh * (d + 4):hh * (d + 4) + d, 0] = u
+            sd[x + "uk"][hh * d:(hh + 1) * d, 0] = u / math.sqrt(5.0)
+        sd[x + "uv"][:, 0] = 3.0 / math.sqrt(5.0)
+    else:
+        sd[x + "lower"][:] = 0.996
+        sd[x + "q"][:, 0] = 1.0
+        sd[x + "v"][:, 1] = 3.0
+    sd = {k: v.to(torch.bfloat16) for k, v in sd.items()}
+    return cfg, sd, lu.write_model(str(tmp_path / f"mark_{kind}"), cfg, sd), mark, vocab
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("kind", ["attention", "latent", "hgrn2"])
+def test_one_token_stands_out_far_back_and_at_page_borders(tmp_path, device, kind):
+    """The marked token at the start, on both sides of page borders and hundreds of places (many pages) back:
+    every later row still depends on it, no earlier one does; seen from prompt rows, from decoded rows, and
+    from the first row after a cut right behind the mark."""
+    cfg, sd, path, mark, vocab = _marked_model(tmp_path, kind)
+    runner = load_runner(path, torch.float32, device, max_tokens=640, max_seqs=2)
+    rng = np.random.default_rng(0)
+    n = 300
+    for place in (0, 15, 16, 31, 32, 143, n - 2):
+        toks = [int(t) for t in rng.integers(8, vocab, n)]
+        toks[place] = mark
+        want = lu.oracle_logits(cfg, sd, toks)
+        plain = lu.oracle_logits(cfg, sd, [t if t != mark else 9 for t in toks])
+        seen = np.array([lu.rel_err(plain[i:i + 1], want[i:i + 1]) for i in range(n)])      # (per row, relative to the row's spread)
+        assert seen[:place].max(initial=0.0) == 0.0
+        assert seen[place + 1:].min() > 100 * TOL, "the marked token does not stand out"
+        assert lu.rel_err(run_cut(runner, "p", toks, [n])[-60:], want[-60:]) < TOL, place
+        cuts = [place + 1] + ([n - 30 - place - 1] if n - 30 - place - 1 > 0 else [])
+        tail = min(60, n - place - 1)
+        assert lu.rel_err(run_cut(runner, "d", toks, cuts)[-tail:], want[-tail:]) < TOL, place
+    runner.close()
+
+
+# ----------------------------------------------------- command line, configuration, graphs, trace replay
+def test_command_line_serves_the_model(tmp_path):
+    from flexible_llm_sharding_amd import api
+    from flexible_llm_sharding_amd.utils.tokenizer import write_synthetic_tokenizer
+    cfg = lu.config(STACK, vocab=64, loop=LOOP)
+    sd = lu.random_weights(cfg, 16)
+    path = lu.write_model(str(tmp_path / "cli"), cfg, sd)
+    write_synthetic_tokenizer(path, 64)
+    prompts = [("w1 w2 w3", ("w4", "w5 w6")), ("w7", ("w8 w9 w10",))]
+    pk = str(tmp_path / "p.pkl")
+    with open(pk, "wb") as f:
+        pickle.dump(prompts, f)
+    out = str(tmp_path / "o.pkl")
+    api.main(["--model_path", path, "--prompt_pickle", pk, "--output_file", out, "--num_gen_token", "3",
+              "--num_gpus", "0" if not gpu_available() else "1", "--dtype", "float32", "--layer_num_per_shard", "2"])
+    with open(out, "rb") as f:
+        scores = pickle.load(f)
+    assert [s.shape for s in scores] == [(2, 3, 64), (1, 3, 64)]
+    assert all(abs(float(s[i, j].astype(np.float32).sum()) - 1) < 2e-2 for s in scores for i in range(s.shape[0]) for j in range(3))
+
+
+def test_config_is_read_not_assumed(tmp_path):
+    """The registry picks the family by config.json's architecture; every pass of a looped layer has a state
+    of its own and shares its layer's weight image; every tensor of the checkpoint lands, none is invented;
+    a checkpoint that contradicts the config is refused at load."""
+    from flexible_llm_sharding_amd.config import LopilixConfig, load_config
+    from flexible_llm_sharding_amd.models import hybrid_family, lopilix
+    from flexible_llm_sharding_amd.runtime.weights import CheckpointSource, HostStore
+    cfg = lu.config(STACK, loop=LOOP)
+    sd = lu.random_weights(cfg, 18)
+    path = lu.write_model(str(tmp_path / "c"), cfg, sd)
+    c = load_config(path)
+    assert isinstance(c, LopilixConfig) and hybrid_family(c) is lopilix
+    assert c.layer_names() == ["embed", "l0", "l1", "l2", "l3", "l1@1", "l2@1", "l3@1", "l4", "final.norm", "head"]
+    assert c.streams == 4 and c.state_width == 4 * 36 and c.residual_mult == 0.7 and c.logit_scale == 0.6 and c.hyper and c.gated
+    spec = lopilix.state_spec(c)
+    assert spec["paged"] == {"l0": {"k": 2 * 2 * 10, "v": 2 * 14}, "l2": {"ckr": 19}, "l2@1": {"ckr": 19}, "l4": {"k": 2 * 3 * 8, "v": 3 * 5}}
+    assert spec["slots"] == {"l1": {"state": (3, 7, 9)}, "l3": {"state": (2, 20, 6)}, "l1@1": {"state": (3, 7, 9)}, "l3@1": {"state": (2, 20, 6)}}
+    names = {pl.hf_name for n in c.layer_names() for pl in lopilix.placements(c, n)}
+    assert names == set(sd)
+    store = HostStore.from_source(CheckpointSource(c, path, torch.float32), pinned=False)
+    assert store.host_buffer("l2@1") is store.host_buffer("l2") and store.host_buffer("l3") is not store.host_buffer("l2")
+    for edit in (lambda d: d["layers"][0].update(type="hyena"),
+                 lambda d: d["layers"][0]["mixer"].update(kv_heads=4),
+                 lambda d: d["layers"][0]["mixer"]["rot"].update(dims=7),
+                 lambda d: d["layers"][2]["mixer"]["rot"].update(dims=10),
+                 lambda d: d["layers"][1]["mlp"]["router"].update(top=9),
+                 lambda d: d["layers"][1]["mlp"]["router"]["groups"].update(count=4),
+                 lambda d: d["layers"][1]["mlp"]["router"]["groups"].update(keep=0),
+                 lambda d: d.update(loop={"start": 2, "stop": 9, "times": 2}),
+                 lambda d: d.update(streams=0)):
+        bad = json.loads(json.dumps(cfg))
+        edit(bad)
+        with pytest.raises((NotImplementedError, ValueError)):
+            LopilixConfig.from_dict(bad)
+    wrong = json.loads(json.dumps(cfg))
+    wrong["layers"][0]["mixer"]["vdim"] = 15
+    lu.write_model(str(tmp_path / "w"), wrong, sd)
+    with pytest.raises(ValueError):
+        load_runner(str(tmp_path / "w"), torch.float32, "cpu")
+
+
+@pytest.mark.gpu
+def test_captured_decode_steps_equal_eager(tmp_path, monkeypatch):
+    """Decode steps replay as captured HIP graphs; every replay is checked against the same steps run
+    eagerly, with eager prompt steps of other requests and batch-size changes between the replays."""
+    if not gpu_available():
+        pytest.skip("no GPU")
+
+    def run(graphs: bool):
+        monkeypatch.setenv("FLS_DECODE_GRAPHS", "1" if graphs else "0")
+        cfg, sd, runner, _ = build(tmp_path, STACK, seed=21, device="cuda:0", dtype=torch.bfloat16, max_tokens=256, max_seqs=4, loop=LOOP)
+        a, b, c = (lu.tokens(n, cfg["vocab"], 60 + n) for n in (40, 33, 25))
+        outs = []
+        runner.step([StepEntry("a", a[:10], [9]), StepEntry("b", b[:12], [11])])
+        for t in range(20):
+            live = [("a", a[10 + t]), ("b", b[12 + t])] + ([("c", c[9 + t - 8])] if t >= 8 else [])
+            r = runner.step([StepEntry(i, [tok], [0]) for i, tok in live])
+            outs += [x[0] for x in r]
+            if t == 7:
+                outs.append(runner.step([StepEntry("c", c[:9], [8])])[0][0])
+            if t % 5 == 0:
+                torch.cuda.synchronize()
+        replays = runner._decode_graphs.replays if runner._decode_graphs is not None else 0
+        runner.close()
+        return np.concatenate(outs, 0), replays
+
+    eager, n0 = run(False)
+    graphed, n1 = run(True)
+    assert n0 == 0 and n1 >= 12
+    assert np.array_equal(eager, graphed)
+
+
+def test_trace_run_program_replays_steps(tmp_path):
+    """bin/trace_run as a process on a two-request schedule: prompts of unequal length in one step,
+    then one token each; a flushed 'done <step>' after each step, logits files for the steps that
+    want some, exit code 0 at end of input."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = lu.config(STACK[:4], vocab=37, loop=(1, 3, 2))
+    sd = lu.random_weights(cfg, 19)
+    path = lu.write_model(str(tmp_path / "t"), cfg, sd)
+    out = tmp_path / "logits"
+    a, b = lu.tokens(9, 37, 4), lu.tokens(3, 37, 5)
+    p = subprocess.Popen([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32",
+                          "--out", str(out), "--max-tokens", "32", "--device", "cpu"], stdin=subprocess.PIPE,
+                         stdout=subprocess.PIPE, text=True, cwd=root)
+    steps = [{"step": 0, "entries": [{"id": "q", "tokens": a[:7], "want": [0, 6]}, {"id": "s", "tokens": b[:1], "want": [0]}], "end": []},
+             {"step": 1, "entries": [{"id": "q", "tokens": a[7:8], "want": []}, {"id": "s", "tokens": b[1:2], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "q", "tokens": a[8:], "want": [0]}, {"id": "s", "tokens": b[2:], "want": [0]}], "end": ["q", "s"]}]
+    for st in steps:
+        p.stdin.write(json.dumps(st) + "\n")
+        p.stdin.flush()
+        while True:
+            line = p.stdout.readline()
+            assert line, "trace_run ended early"
+            if line.strip() == f"done {st['step']}":
+                break
+    p.stdin.close()
+    assert p.wait(timeout=60) == 0
+    wa, wb = lu.oracle_logits(cfg, sd, a), lu.oracle_logits(cfg, sd, b)
+    got = np.concatenate([np.fromfile(out / "0.f32", dtype="<f4").reshape(3, -1), np.fromfile(out / "2.f32", dtype="<f4").reshape(2, -1)])
+    assert not (out / "1.f32").exists()
+    assert lu.rel_err(got, np.concatenate([wa[[0, 6]], wb[[0]], wa[[8]], wb[[2]]])) < TOL

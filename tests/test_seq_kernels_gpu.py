@@ -535,3 +535,138 @@ def test_residual_add_with_the_next_norm(ops, cdt, tol):
         ha, hb = H.add_scaled_dyt_norm_(a, y, 0.6, wb, alpha, cdt), R.add_scaled_dyt_norm_(b, y, 0.6, wb, alpha, cdt)
         close(a, b, 1e-6)
         close(ha, hb, tol)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("S,D", [(1, 36), (3, 320), (5, 34), (2, 2304)])
+def test_residual_streams_norm_update_and_embedding_copies(ops, cdt, tol, S, D):
+    """Several residual streams side by side in a row: their weighted sum through the RMS norm (also the plain
+    sum with a row gather), the update of all streams at once with the gated sublayer output (gate logits as a
+    column block of a wider matrix), the same fused with the next norm, one stream without coefficients, and the
+    embedding with a position vector written S times."""
+    H, R = ops
+    torch.manual_seed(S * D)
+    T = 37
+    xs = torch.randn(T, S * D, device=DEV)
+    hc = torch.randn(2 * S + S * S, device=DEV)
+    w = 1 + 0.3 * torch.randn(D, device=DEV)
+    idx = torch.tensor([5, 0, 36, 5], dtype=torch.int32, device=DEV)
+    close(H.streams_norm(xs, hc, w, 1e-5, cdt, S), R.streams_norm(xs, hc, w, 1e-5, cdt, S), tol)
+    close(H.streams_norm(xs, None, w, 1e-5, cdt, S, row_idx=idx), R.streams_norm(xs, None, w, 1e-5, cdt, S, row_idx=idx), tol)
+    y = torch.randn(T, D, device=DEV)
+    z = torch.randn(T, D + 24, device=DEV)
+    gate = z[:, 8:8 + D]
+    for g in (gate, None):
+        a, b = xs.clone(), xs.clone()
+        close(H.streams_update_(a, y, g, hc, 0.45, S), R.streams_update_(b, y, g, hc, 0.45, S), 1e-5)
+        a, b = xs.clone(), xs.clone()
+        hc2 = torch.randn(2 * S + S * S, device=DEV)
+        close(H.streams_update_norm_(a, y, g, hc, 0.45, S, hc2, w, 1e-5, cdt), R.streams_update_norm_(b, y, g, hc, 0.45, S, hc2, w, 1e-5, cdt), tol)
+        close(a, b, 1e-5)
+    if S == 1:
+        a, b = xs.clone(), xs.clone()
+        close(H.streams_update_norm_(a, y, gate, None, 0.7, 1, None, w, 1e-5, cdt), R.streams_update_norm_(b, y, gate, None, 0.7, 1, None, w, 1e-5, cdt), tol)
+        close(a, b, 1e-5)
+    table, ptab = torch.randn(50, D, device=DEV).to(cdt), torch.randn(90, D, device=DEV).to(cdt)
+    ids = torch.randint(0, 50, (T,), dtype=torch.int32, device=DEV)
+    pos = torch.randint(0, 90, (T,), dtype=torch.int32, device=DEV)
+    close(H.embed_rows(ids, table, pos_table=ptab, tok_pos=pos, copies=S), R.embed_rows(ids, table, pos_table=ptab, tok_pos=pos, copies=S), 1e-6)
+    close(H.embed_rows(ids, table, scale=1.5, copies=S), R.embed_rows(ids, table, scale=1.5, copies=S), 1e-6)
+    lg = torch.randn(T, 70, device=DEV)
+    close(H.scale_(lg.clone(), 0.25), R.scale_(lg.clone(), 0.25), 1e-7)
+    o = torch.randn(T, D, device=DEV)
+    close(H.sigmoid_gate(o, y, cdt), R.sigmoid_gate(o, y, cdt), tol)
+    close(H.sigmoid_gate(o.to(cdt), y, cdt), R.sigmoid_gate(o.to(cdt), y, cdt), tol)
+    close(H.unary(o, "gelu", cdt), R.unary(o, "gelu", cdt), tol)
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+def test_rotation_in_halves_with_turn_count_rescaling(ops, cdt, tol):
+    """Pairs (i, i + dims / 2) with frequencies rescaled by turn counts and amplified cosines and sines, with and
+    without the norm in front, over part of a head and over heads wider than a wave, into a pool and in place."""
+    H, R = ops
+    torch.manual_seed(4)
+    md, n_pages, _ = meta_of([40, 3, 1], [0, 77, 1200], DEV)
+    T = 44
+    sc = ("turns", 3.0, 300.0, 20.0, 2.0)
+    for heads, n, dims in ((3, 32, 32), (2, 24, 10), (1, 200, 160), (4, 8, 8)):
+        x = torch.randn(T, heads * n + 6, device=DEV)
+        w = 1 + 0.2 * torch.randn(n, device=DEV)
+        for ww in (w, None):
+            a, b = torch.zeros(T, heads * n, device=DEV, dtype=cdt), torch.zeros(T, heads * n, device=DEV, dtype=cdt)
+            kw = dict(w=ww, eps=1e-5, rot=(dims, 1e4, sc), half=True)
+            close(H.head_norm_rope(x, heads, n, 3, n, a, 0, n, md, **kw), R.head_norm_rope(x, heads, n, 3, n, b, 0, n, md, **kw), tol)
+        pa = torch.zeros(n_pages * 16, n + 5, device=DEV, dtype=cdt)
+        pb = pa.clone()
+        kw = dict(rot=(dims, 1e4, sc), half=True, row_map=md["kv_slot"])
+        close(H.head_norm_rope(x, 1, n, 0, 0, pa, 5, 0, md, **kw), R.head_norm_rope(x, 1, n, 0, 0, pb, 5, 0, md, **kw), tol)
+        xa, xb = x.clone(), x.clone()                                   # in place: every pair is read before it is written
+        kw = dict(rot=(dims, 50.0), half=True)
+        close(H.head_norm_rope(xa, heads, dims, n - dims, n, xa, n - dims, n, md, **kw), R.head_norm_rope(xb, heads, dims, n - dims, n, xb, n - dims, n, md, **kw), 1e-5)
+    f = R.rope_freqs(32, 1e6, "cpu", sc)
+    f0 = R.rope_freqs(32, 1e6, "cpu")
+    assert f[0] == f0[0] and abs(float(f[-1] / f0[-1]) - 1 / 3) < 1e-6 and abs(R.rope_amp(sc) - (0.1 * np.log(3.0) + 1)) < 1e-12
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("Hh,G,d,dv", [(6, 2, 10, 14), (2, 2, 32, 48), (4, 2, 64, 128), (2, 1, 128, 64)])
+def test_two_score_maps_over_shared_values_and_their_combine(ops, cdt, tol, Hh, G, d, dv):
+    """Differential attention's pieces: 2 H query heads over 2 G key heads whose value head is the key head
+    modulo G, fp32 outputs over pools of the GEMM type (prompt rows over tiles and decoded rows over long
+    contexts with split keys), then the combine a1 - lambda a2 with its unit norm."""
+    H, R = ops
+    torch.manual_seed(Hh * d)
+    for lens, pos0 in (([150, 17], [0, 0]), ([1, 1], [700, 45]), ([5, 40], [3, 90])):
+        md, n_pages, _ = meta_of(lens, pos0, DEV)
+        T = sum(lens)
+        kc = (torch.randn(n_pages, 16, 2 * G * d, device=DEV) * 0.5).to(cdt)
+        vc = torch.randn(n_pages, 16, G * dv, device=DEV).to(cdt)
+        q = torch.randn(T, 2 * Hh * d, device=DEV)
+        kw = dict(scale=d ** -0.5, softcap=0.0, r1=None, r2=None, chunk=0, page_size=16, out_dtype=cdt, v_heads=G)
+        a, b = torch.empty(T, 2 * Hh * dv, device=DEV), torch.empty(T, 2 * Hh * dv, device=DEV)
+        H.attn_paged(q, kc, vc, md, 2 * Hh, 2 * G, d, dv, out=a, **kw)
+        R.attn_paged(q, kc, vc, md, 2 * Hh, 2 * G, d, dv, out=b, **kw)
+        close(a, b, 2e-5 if cdt == torch.float32 else 1e-2)
+        lam = 0.4 * torch.randn(4, d, device=DEV)
+        close(H.diff_combine(b, lam, 0.35, Hh, dv, 1e-6, cdt), R.diff_combine(b, lam, 0.35, Hh, dv, 1e-6, cdt), tol)
+
+
+@pytest.mark.parametrize("heads,dim,vdim", [(3, 7, 9), (5, 48, 72), (1, 1, 1), (2, 130, 70), (4, 128, 128), (1, 256, 300)])
+def test_hgrn2_scan_carries_state(ops, heads, dim, vdim):
+    """The gated recurrence over a batch of unequal requests, some continuing from carried states in scattered
+    slots (prompt portions and single decoded rows), with and without the gate's bias; outputs and states."""
+    H, R = ops
+    torch.manual_seed(heads + dim)
+    for lens, pos0 in (([33, 1, 7], [0, 5, 12]), ([1, 1, 1], [4, 0, 9]), ([70], [0])):
+        md, _, n_slots = meta_of(lens, pos0, DEV)
+        T = sum(lens)
+        z = torch.randn(T, 2 * heads * dim + heads * vdim + 5, device=DEV)
+        q, f, v = z[:, :heads * dim], z[:, heads * dim:2 * heads * dim], z[:, 2 * heads * dim:2 * heads * dim + heads * vdim]
+        fb = torch.randn(heads * dim, device=DEV)
+        lower = torch.rand(heads * dim, device=DEV)
+        nw = 1 + 0.2 * torch.randn(vdim, device=DEV)
+        st = torch.randn(n_slots, heads, dim, vdim, device=DEV)
+        for bias in (fb, None):
+            s1, s2 = st.clone(), st.clone()
+            a = H.hgrn2_scan(q, f, v, bias, lower, nw, s1, md, heads, dim, vdim, 1e-5, torch.float32)
+            b = R.hgrn2_scan(q, f, v, bias, lower, nw, s2, md, heads, dim, vdim, 1e-5, torch.float32)
+            close(a, b, 2e-4)
+            close(s1[md["slot"].long()], s2[md["slot"].long()], 2e-4)
+
+
+@pytest.mark.parametrize("T,E,top,groups,keep", [(50, 8, 2, 4, 3), (7, 12, 3, 4, 2), (300, 5, 2, 5, 3), (33, 6, 6, 2, 2), (20, 7, 1, 0, 0),
+                                                 (64, 64, 8, 8, 4), (9, 128, 16, 64, 9)])
+def test_grouped_sigmoid_routing(ops, T, E, top, groups, keep):
+    H, R = ops
+    torch.manual_seed(T + E)
+    logits = torch.randn(T, E + 3, device=DEV)[:, 1:1 + E] * 2
+    a, b = H.moe_route_grouped(logits, top, groups, keep, 1.9), R.moe_route_grouped(logits, top, groups, keep, 1.9)
+    assert torch.equal(a.ids.cpu().sort(-1).values, b.ids.cpu().sort(-1).values)
+    assert torch.equal(a.ids.cpu(), b.ids.cpu())
+    close(a.w, b.w, 1e-5)
+    assert torch.equal(a.offs.cpu(), b.offs.cpu())
+    assert torch.equal(a.rows.cpu().long().bincount(minlength=T), torch.full((T,), top))
+    # every (token, choice) sits in its expert's range of sorted rows
+    offs, dest = a.offs.cpu().long(), a.dest.cpu().long()
+    assert bool(((dest >= offs[a.ids.cpu().long()]) & (dest < offs[a.ids.cpu().long() + 1])).all())
+    assert torch.equal(a.rows.cpu().long()[dest], torch.arange(T)[:, None].expand(T, top))
