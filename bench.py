@@ -149,8 +149,8 @@ def parse(argv=None):
     ap.add_argument("--hybrid", default=None, choices=["s", "m"],
                     help="instead of the headline: prefill / decode throughput of a Kagolix hybrid stack of this size, "
                          "of a Mixtral-structured stack of equal size, and each hybrid kernel alone (one GPU)")
-    ap.add_argument("--hybrid-family", default="kagolix", choices=["kagolix", "sisavik", "gizezen"],
-                    help="with --hybrid: the family to measure (sisavik, gizezen: beside a Kagolix stack of equal size)")
+    ap.add_argument("--hybrid-family", default="kagolix", choices=["kagolix", "sisavik", "gizezen", "lopilix"],
+                    help="with --hybrid: the family to measure (sisavik, gizezen, lopilix: beside a Kagolix stack of equal size)")
     ap.add_argument("--hybrid-dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--hybrid-batch", type=int, default=8)
     ap.add_argument("--hybrid-context", type=int, default=2048)

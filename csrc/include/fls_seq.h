@@ -101,11 +101,14 @@ int fls_seq_causal_conv(const float* x, int ldx, const float* w, const float* b,
 // projected rows z = [q (H d) | k (G d) | v (G dv) | ...] into attention in one pass: causal convolution per channel
 // (w [C, taps] nullable, history in state[slot][taps-1][C] as for fls_seq_causal_conv), q and k heads rotated in pairs
 // over their first rot entries (angle tok_pos * freqs[i]) and divided by sqrt(mean(head^2) + eps), q to qo (fp32
-// [T, H d]), k and v (v as convolved) to row kv_slot[t] of pools of type tc.  G = 0: queries only.  d, dv <= 512
+// [T, H d]), k and v (v as convolved) to row kv_slot[t] of pools of type tc.  G = 0: queries only.  d, dv <= 512.
+// Gv (< 0: G): the row holds Gv value heads after its G key heads.  qnw / knw (nullable, [d]): the q / k heads are instead
+// RMS-normed BEFORE the rotation, times that weight (x / rms(x) * w, then rotated).
 int fls_seq_qkv_conv_rope(const float* z, int ldz, const float* w, float* state, int taps, const int* tok_seq,
                           const int* tok_pos, const int* cu, const int* pos0, const int* slot, const int* kv_slot,
                           int T, int B, int H, int G, int d, int dv, float eps, const float* freqs, int rot, float* qo,
-                          int ldq, void* kc, int ldk, void* vc, int ldv, int tc, int one_row_each, fls_stream_t s);
+                          int ldq, void* kc, int ldk, void* vc, int ldv, int tc, int one_row_each, int Gv, const float* qnw,
+                          const float* knw, fls_stream_t s);
 // generalized delta rule, per head a state S[d][d] in state[slot][H][d][d]:
 // S_t = diag(w) S_(t-1) - (a * u)(u^T S_(t-1)) + k v^T, o = S_t^T r; u = k / sqrt(sum k^2 + key_eps),
 // w = exp(-decay_scale sigmoid(wz + w0)), a = sigmoid(az); out = out_scale o / rms_head(o; norm_eps) norm_w sigmoid(g).

@@ -158,10 +158,11 @@ __global__ __launch_bounds__(256) void qkv_conv_rope_kernel(const float* __restr
                                                             const int* __restrict__ kv_slot, int H, int G, int d, int dv, float eps,
                                                             const float* __restrict__ freqs, int rot, float* __restrict__ qo,
                                                             int ldq, TO* __restrict__ kc, int ldk, TO* __restrict__ vc, int ldv,
-                                                            int C, int fuse_state) {
+                                                            int C, int fuse_state, int Gv, const float* __restrict__ qnw,
+                                                            const float* __restrict__ knw) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x;
-  const int ipr = H + 2 * G;
+  const int ipr = H + G + Gv;
   const int s = tok_seq[t];
   const int tl = t - cu[s];
   const bool carried = pos0[s] > 0;
@@ -242,12 +243,23 @@ __global__ __launch_bounds__(256) void qkv_conv_rope_kernel(const float* __restr
       continue;
     }
     float s2 = 0.f;
+    // a weighted norm comes before the rotation: the root mean square of the entries as they are, the weight on every
+    // entry, then the rotation (which the scalar 1 / rms passes through); without a weight the unit norm follows the rotation
+    const float* nw = kind == 0 ? qnw : knw;         // (wave-uniform)
+    if (nw != nullptr) {
+#pragma unroll
+      for (int e = 0; e < NE; ++e) {
+        const int c = lane + 64 * e;
+        s2 += v[e] * v[e];
+        v[e] *= c < n ? nw[c] : 0.f;
+      }
+    }
 #pragma unroll
     for (int e = 0; e < NE; ++e) {
       const int c = lane + 64 * e;
       const float other = __shfl_xor(v[e], 1, 64);
       if (c < rot) v[e] = (c & 1) ? v[e] * cs[e] + other * sn[e] : v[e] * cs[e] - other * sn[e];
-      s2 += v[e] * v[e];                              // (entries past n are zeros)
+      if (nw == nullptr) s2 += v[e] * v[e];           // (entries past n are zeros)
     }
     const float rs = 1.f / sqrtf(wave_sum(s2) / (float)n + eps);
     if (kind == 0) {
@@ -266,9 +278,10 @@ template <typename TO>
 static void qkv_launch(int TP, int ne, dim3 grid, hipStream_t st, const float* z, int ldz, const float* w, float* state, int taps,
                        const int* tok_seq, const int* tok_pos, const int* cu, const int* pos0, const int* slot, const int* kv_slot,
                        int H, int G, int d, int dv, float eps, const float* freqs, int rot, float* qo, int ldq, TO* kc, int ldk,
-                       TO* vc, int ldv, int C, int fuse) {
+                       TO* vc, int ldv, int C, int fuse, int Gv, const float* qnw, const float* knw) {
 #define QKV_GO(TT, NN) hipLaunchKernelGGL((qkv_conv_rope_kernel<TO, TT, NN>), grid, dim3(256), 0, st, z, ldz, w, state, taps, tok_seq, \
-                                          tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, kc, ldk, vc, ldv, C, fuse)
+                                          tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, kc, ldk, vc, ldv, C, fuse, \
+                                          Gv, qnw, knw)
 #define QKV_NE(TT) do { if (ne <= 1) QKV_GO(TT, 1); else if (ne <= 2) QKV_GO(TT, 2); else QKV_GO(TT, QKV_MAX_E); } while (0)
   if (TP == 2) QKV_NE(2);
   else if (TP == 3) QKV_NE(3);
@@ -281,15 +294,17 @@ static void qkv_launch(int TP, int ne, dim3 grid, hipStream_t st, const float* z
 extern "C" int fls_seq_qkv_conv_rope(const float* z, int ldz, const float* w, float* state, int taps, const int* tok_seq,
                                      const int* tok_pos, const int* cu, const int* pos0, const int* slot, const int* kv_slot,
                                      int T, int B, int H, int G, int d, int dv, float eps, const float* freqs, int rot, float* qo,
-                                     int ldq, void* kc, int ldk, void* vc, int ldv, int tc, int one_row_each, fls_stream_t s) {
+                                     int ldq, void* kc, int ldk, void* vc, int ldv, int tc, int one_row_each, int Gv,
+                                     const float* qnw, const float* knw, fls_stream_t s) {
   if (T <= 0) return 0;
+  if (Gv < 0 || G == 0) Gv = G;
   if (H < 1 || G < 0 || d < 1 || d > 64 * QKV_MAX_E || dv > 64 * QKV_MAX_E || rot < 0 || rot > d || (rot & 1) ||
       (rot > 0 && freqs == nullptr) || (G > 0 && (kc == nullptr || vc == nullptr || kv_slot == nullptr || dv < 1)) ||
       (w != nullptr && (taps < 1 || (taps > 1 && state == nullptr))))
     return -1;
-  const int C = H * d + G * (d + dv);
-  if (C > ldz || H * d > ldq || (G > 0 && (G * d > ldk || G * dv > ldv))) return -1;
-  const int ipr = H + 2 * G;
+  const int C = H * d + G * d + Gv * dv;
+  if (C > ldz || H * d > ldq || (G > 0 && (G * d > ldk || Gv * dv > ldv))) return -1;
+  const int ipr = H + G + Gv;
   // blocks per row: one when the rows alone fill the chip (every wave then reuses its sines and cosines for a
   // quarter of the row's heads), up to a wave per head when rows are few
   const int per_row_max = (ipr + 3) / 4;
@@ -300,8 +315,8 @@ extern "C" int fls_seq_qkv_conv_rope(const float* z, int ldz, const float* w, fl
   hipStream_t st = (hipStream_t)s;
   const int TP = (w != nullptr && taps >= 2 && taps <= 4) ? taps : 0;
   const int ne = ((d > dv ? d : dv) + 63) / 64;
-  if (tc == 1) qkv_launch<bf16_t>(TP, ne, grid, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (bf16_t*)kc, ldk, (bf16_t*)vc, ldv, C, fuse);
-  else qkv_launch<float>(TP, ne, grid, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (float*)kc, ldk, (float*)vc, ldv, C, fuse);
+  if (tc == 1) qkv_launch<bf16_t>(TP, ne, grid, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (bf16_t*)kc, ldk, (bf16_t*)vc, ldv, C, fuse, Gv, qnw, knw);
+  else qkv_launch<float>(TP, ne, grid, st, z, ldz, w, state, taps, tok_seq, tok_pos, cu, pos0, slot, kv_slot, H, G, d, dv, eps, freqs, rot, qo, ldq, (float*)kc, ldk, (float*)vc, ldv, C, fuse, Gv, qnw, knw);
   SEQ_LAUNCH_CHECK();
   if (w != nullptr && taps > 1 && !fuse) {
     hipLaunchKernelGGL(conv_state_kernel, dim3((C + 255) / 256, B), dim3(256), 0, st, z, ldz, state, cu, pos0, slot, C, taps);

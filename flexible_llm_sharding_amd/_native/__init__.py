@@ -146,7 +146,7 @@ def _load_seq():
     _bind(lib, "fls_seq_dyt_norm", i, p, i, p, p, p, p, i, i, i, i, p)
     _bind(lib, "fls_seq_add_scaled", i, p, i, p, i, i, i, f, p)
     _bind(lib, "fls_seq_add_scaled_dyt", i, p, i, p, i, f, p, p, p, i, i, i, i, p)
-    _bind(lib, "fls_seq_qkv_conv_rope", i, p, i, p, p, i, p, p, p, p, p, p, i, i, i, i, i, i, f, p, i, p, i, p, i, p, i, i, i, p)
+    _bind(lib, "fls_seq_qkv_conv_rope", i, p, i, p, p, i, p, p, p, p, p, p, i, i, i, i, i, i, f, p, i, p, i, p, i, p, i, i, i, i, p, p, p)
     _bind(lib, "fls_seq_moe_combine", i, p, i, p, i, p, p, i, i, p, i, p, i, i, f, p)
     _bind(lib, "fls_seq_gather_rows", i, p, i, i, p, p, i, i, i, p)
     _bind(lib, "fls_seq_xielu", i, p, i, p, p, i, i, i, i, p)

@@ -770,7 +770,11 @@ class LopilixConfig:
     hidden_size = KagolixConfig.hidden_size
     vocab_size = KagolixConfig.vocab_size
     save = KagolixConfig.save
-    total_params = KagolixConfig.total_params
+
+    def total_params(self) -> int:
+        from .models.layout import layer_image, layer_layout_of
+        images = dict.fromkeys(layer_image(n) for n in self.layer_names() if n != "head")     # (the head is the embedding table)
+        return sum(sum(s.numel for s in layer_layout_of(self, n).slots) for n in images)
 
     @property
     def state_width(self) -> int:

@@ -255,11 +255,18 @@ class HipSeqOps:
              "fls_seq_moe_place")
         return SeqRoute(ids, w, offs, rows, dest, top)
 
-    def qkv_conv_rope_store(self, z, w, state, meta, H, G, d, dv, q_out, kc, vc, eps=0.0, rot=None):
+    def qkv_conv_rope_store(self, z, w, state, meta, H, G, d, dv, q_out, kc, vc, eps=0.0, rot=None, v_heads=None, q_norm=None,
+                            k_norm=None):
         _rows(z, "z", torch.float32)
         _rows(q_out, "q_out", torch.float32)
         T = z.shape[0]
-        C = H * d + G * (d + dv)
+        Gv = G if v_heads is None else int(v_heads)
+        C = H * d + G * d + Gv * dv
+        for nme, t in (("q_norm", q_norm), ("k_norm", k_norm)):
+            if t is not None:
+                _vec(t, nme, d)
+        if (q_norm is None) != (k_norm is None) and G:
+            raise ValueError("qkv_conv_rope_store: q_norm and k_norm come together")
         if z.shape[1] < C or tuple(q_out.shape) != (T, H * d):
             raise ValueError("qkv_conv_rope_store: rows do not fit the head sizes")
         taps = 1
@@ -271,7 +278,7 @@ class HipSeqOps:
                 raise ValueError("qkv_conv_rope_store: state must be fp32 [slots, taps - 1, C]")
         tc = 0
         if G:
-            if kc.dtype != vc.dtype or kc.shape[-1] < G * d or vc.shape[-1] < G * dv or not kc.is_contiguous() \
+            if kc.dtype != vc.dtype or kc.shape[-1] < G * d or vc.shape[-1] < Gv * dv or not kc.is_contiguous() \
                     or not vc.is_contiguous():
                 raise ValueError("qkv_conv_rope_store: pools do not fit the head sizes")
             tc = _code(kc, "kc")
@@ -288,7 +295,9 @@ class HipSeqOps:
                                           freqs.data_ptr() if freqs is not None else None, dims, q_out.data_ptr(),
                                           q_out.stride(0), kc.data_ptr() if G else None, kc.shape[-1] if G else 0,
                                           vc.data_ptr() if G else None, vc.shape[-1] if G else 0, tc,
-                                          1 if meta.get("max_rows") == 1 else 0, _stream()), "fls_seq_qkv_conv_rope")
+                                          1 if meta.get("max_rows") == 1 else 0, Gv,
+                                          q_norm.data_ptr() if q_norm is not None else None,
+                                          k_norm.data_ptr() if k_norm is not None else None, _stream()), "fls_seq_qkv_conv_rope")
         return q_out
 
     def _gemm(self, a, w, c, bias, M, N, K, lda, ldw, ldc, groups=1, offs=None, a_gs=0, a_mod=1, w_gs=0, c_gs=0,

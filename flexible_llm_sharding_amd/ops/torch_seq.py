@@ -248,25 +248,29 @@ class TorchSeqOps:
                 raw[rows, out_col + h * out_hs:out_col + h * out_hs + n] = keep[:, h].to(raw.dtype)
         return out
 
-    def qkv_conv_rope_store(self, z, w, state, meta, H, G, d, dv, q_out, kc, vc, eps=0.0, rot=None):
+    def qkv_conv_rope_store(self, z, w, state, meta, H, G, d, dv, q_out, kc, vc, eps=0.0, rot=None, v_heads=None, q_norm=None,
+                            k_norm=None):
         """The projected rows z = [q (H d) | k (G d) | v (G dv) | ...] of a step on their way into attention:
         a short causal convolution per channel (``w`` [C, taps], no bias; the last taps - 1 rows of a request
         carried in ``state[slot]``, None for one tap), then for q and k heads the pair rotation ``rot`` and
         the division by the head's root mean square (eps inside the root), v as convolved.  q goes to
         ``q_out`` [T, H d] fp32, k and v to the rows ``kv_slot`` of their pools.  G = 0 (kc, vc None): a layer
-        that reads another layer's keys and values has only queries."""
-        C = H * d + G * (d + dv)
+        that reads another layer's keys and values has only queries.  ``v_heads``: the row holds that many value
+        heads (instead of G) behind its G key heads.  ``q_norm`` / ``k_norm`` ([d]): the q / k heads are instead
+        RMS-normed before the rotation and multiplied by that weight."""
+        Gv = G if v_heads is None else int(v_heads)
+        C = H * d + G * d + Gv * dv
         u = z[:, :C]
         if w is not None:
             if w.shape[1] > 1:
                 u = self.causal_conv(u, w, None, state, meta)
             else:
                 u = u.float() * w.float()[:, 0]
-        self.head_norm_rope(u, H, d, 0, d, q_out, 0, d, meta, eps=eps, rot=rot, unit_after=True)
+        self.head_norm_rope(u, H, d, 0, d, q_out, 0, d, meta, w=q_norm, eps=eps, rot=rot, unit_after=q_norm is None)
         if G:
-            self.head_norm_rope(u, G, d, H * d, d, kc.view(-1, kc.shape[-1]), 0, d, meta, eps=eps, rot=rot, unit_after=True,
-                                row_map=meta["kv_slot"])
-            self.head_norm_rope(u, G, dv, (H + G) * d, dv, vc.view(-1, vc.shape[-1]), 0, dv, meta, row_map=meta["kv_slot"])
+            self.head_norm_rope(u, G, d, H * d, d, kc.view(-1, kc.shape[-1]), 0, d, meta, w=k_norm, eps=eps, rot=rot,
+                                unit_after=k_norm is None, row_map=meta["kv_slot"])
+            self.head_norm_rope(u, Gv, dv, (H + G) * d, dv, vc.view(-1, vc.shape[-1]), 0, dv, meta, row_map=meta["kv_slot"])
         return q_out
 
     def softcap_(self, z, cap):

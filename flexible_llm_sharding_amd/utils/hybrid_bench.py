@@ -1,6 +1,7 @@
 """Throughput of a hybrid stack next to the closest existing model at equal size: ``bench.py --hybrid``
 (Kagolix beside a Mixtral-structured stack; ``--hybrid-family sisavik``: Sisavik beside Kagolix;
-``--hybrid-family gizezen``: Gizezen beside a Kagolix stack of attention layers with experts).
+``--hybrid-family gizezen``: Gizezen beside a Kagolix stack of attention layers with experts;
+``--hybrid-family lopilix``: Lopilix beside the Kagolix stack of attention, recurrent and state-space layers).
 
 Random weights at sizes that resemble a real model's layers.  Three parts, one JSON line each:
 
@@ -21,7 +22,7 @@ from typing import Dict, List
 import numpy as np
 import torch
 
-from ..config import GizezenConfig, KagolixConfig, ModelConfig, SisavikConfig
+from ..config import GizezenConfig, KagolixConfig, LopilixConfig, ModelConfig, SisavikConfig
 
 PEAK_FLOPS = 2.5e15        # dense bf16 / fp16 matrix peak of one MI355X
 PEAK_BYTES = 8.0e12        # HBM3E
@@ -96,6 +97,26 @@ def gizezen_config(z: dict, repeats: int = 3) -> GizezenConfig:
                                     "residual_mult": 0.6, "embedding": {"scale": 1.5}, "layers": layers})
 
 
+def lopilix_config(z: dict, times: int = 2, streams: int = 4) -> LopilixConfig:
+    """Differential attention with a dense feed-forward, HGRN2 with experts, latent attention with experts; the
+    three layers run ``times`` times in a row on the same weights (six layer runs), over ``streams`` residual
+    streams.  Head sizes, ranks and expert sizes of the order real models use."""
+    d = z["dim"]
+    att = {"heads": z["heads"], "kv_heads": z["kv"], "dim": d // 2, "vdim": d, "rot": {"dims": d // 2, "base": 5.0e5},
+           "scale": (d // 2) ** -0.5, "diff": 0.2}
+    rec = {"heads": z["width"] // d, "dim": d, "vdim": d}
+    lat = {"heads": z["heads"], "dim": d // 2, "rot_dim": d // 2, "vdim": d, "kv_rank": 4 * d, "scale": d ** -0.5,
+           "rot": {"dims": d // 2, "base": 5.0e5, "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}
+    dense = {"kind": "dense", "ff": z["ff"] * 2 // 3 // 64 * 64}        # (gated: three matrices instead of two)
+    moe = {"kind": "moe", "expert": {"ff": z["eff"]},
+           "router": {"experts": z["experts"], "top": z["top"], "scale": 2.0, "groups": {"count": z["experts"] // 2, "keep": z["experts"] // 4}}}
+    layers = [{"type": "attention", "mixer": att, "mlp": dense}, {"type": "hgrn2", "mixer": rec, "mlp": moe},
+              {"type": "latent_attention", "mixer": lat, "mlp": moe}]
+    return LopilixConfig.from_dict({"architecture": "Lopilix", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6},
+                                    "residual_mult": 0.5, "streams": streams, "logit_scale": 0.5, "max_positions": 8192,
+                                    "loop": {"start": 0, "stop": 3, "times": times}, "layers": layers})
+
+
 def kagolix_attention_moe_config(z: dict, n_layers: int = 6) -> KagolixConfig:
     """The Kagolix stack a Gizezen stack is measured against: chunk-local attention and routed experts in
     every layer (the same heads, head size, experts and expert width; no shared expert, no shared keys)."""
@@ -131,6 +152,12 @@ def synthetic_hybrid_store(cfg: KagolixConfig, device, dtype, seed: int = 0):
             elif cfg.family == "gizezen" and k.startswith("norm"):
                 v[0].copy_(1.0 + 0.1 * torch.randn(v.shape[1:], generator=g, device=device))    # [weight; bias]
                 v[1].copy_(0.1 * torch.randn(v.shape[1:], generator=g, device=device))
+            elif cfg.family == "lopilix" and k.startswith("hc"):
+                S = cfg.streams                                       # [in | out | mix]: an even read, a unit write, streams that keep themselves
+                v.copy_(torch.cat([torch.full((S,), 1.0 / S), torch.ones(S), torch.eye(S).reshape(-1)]).to(device)
+                        + 0.05 * torch.randn(v.shape, generator=g, device=device))
+            elif k == "lower":
+                v.copy_(0.9 * torch.rand(v.shape, generator=g, device=device))
             elif k.startswith("alpha"):
                 v.fill_(0.5)
             elif k.startswith("norm") or k in ("qn", "kn", "mnorm", "dqn", "dkvn", "lqn", "lkn", "rnorm"):
@@ -542,6 +569,151 @@ def bench_gizezen_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
     return {"part": "kernels", "family": "gizezen", "dtype": str(dtype), "batch": B, "context": L, "kernels": res}
 
 
+def bench_lopilix_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
+    """The kernels of the Lopilix layers alone at the prefill shape (T = B L rows) and the decode shape (B rows at
+    context L), each beside the like kernel of the Kagolix family on a like shape."""
+    from ..models.lopilix import _rot
+    from ..ops import get_ops
+    ops = get_ops(dev, dtype, family="hybrid")
+    es = 2 if dtype == torch.bfloat16 else 4
+    cfg = lopilix_config(z, 1)
+    att, rc, lat = (l.mixer for l in cfg.layers)
+    mlp = cfg.layers[1].mlp
+    D, S, ps = z["width"], cfg.streams, 16
+    H, G, d, dv = att["heads"], att["kv_heads"], att["dim"], att["vdim"]
+    E, top, ff = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"]
+    res: Dict[str, dict] = {}
+
+    def rec(name, sec, flops=0.0, nbytes=0.0):
+        e = {"us": sec * 1e6}
+        if flops:
+            e["tflops"] = flops / sec / 1e12
+            e["of_matrix_peak"] = flops / sec / PEAK_FLOPS
+        if nbytes:
+            e["gb_s"] = nbytes / sec / 1e9
+            e["of_hbm"] = nbytes / sec / PEAK_BYTES
+        res[name] = {k: round(v, 4) for k, v in e.items()}
+
+    for tag, lens, pos0 in (("prefill", [L] * B, [0] * B), ("decode", [1] * B, [L - 1] * B)):
+        T = sum(lens)
+        meta = step_meta(B, lens, pos0, L, dev, ps)
+        meta["max_rows"] = max(lens)
+        pos = meta["pos_host"]
+        reps = 5 if tag == "prefill" else 30
+        keys = float(np.mean([p + 1 for p in pos]))
+        # two score maps over shared values (2 H heads over 2 G key heads, fp32 out) | Kagolix: chunk-local softmax attention
+        kc = torch.randn(meta["n_pages"], ps, 2 * G * d, device=dev).to(dtype)
+        vc = torch.randn(meta["n_pages"], ps, G * dv, device=dev).to(dtype)
+        q = torch.randn(T, 2 * H * d, device=dev)
+        a = torch.empty(T, 2 * H * dv, device=dev)
+        rec(f"{tag}/differential attention, two maps", _timed(lambda: ops.attn_paged(
+            q, kc, vc, meta, 2 * H, 2 * G, d, dv, d ** -0.5, 0.0, None, None, 0, ps, dtype, out=a, v_heads=G), reps),
+            2.0 * T * keys * 2 * H * (d + dv), 0 if tag == "prefill" else B * keys * (2 * G * d + G * dv) * es)
+        dk = z["dim"]
+        kk = torch.randn(meta["n_pages"], ps, G * dk, device=dev).to(dtype)
+        qk = torch.randn(T, H * dk, device=dev).to(dtype)
+        r1 = torch.rand(H, device=dev)
+        keys_k = float(np.mean([p % z["chunk"] + 1 for p in pos]))
+        rec(f"kagolix {tag}/chunk attention", _timed(lambda: ops.attn_paged(qk, kk, kk, meta, H, G, dk, dk, dk ** -0.5, 30.0, r1, r1,
+                                                                              z["chunk"], ps, dtype), reps),
+            4.0 * T * keys_k * H * dk, 0 if tag == "prefill" else 2.0 * B * keys_k * G * dk * es)
+        lam = 0.1 * torch.randn(4, d, device=dev)
+        rec(f"{tag}/differential combine + unit norm", _timed(lambda: ops.diff_combine(a, lam, 0.2, H, dv, 1e-6, dtype), reps), 0,
+            T * H * dv * (8 + es))
+        # q and k: norm per head and map, rotation, page write; v: page write | Kagolix: query norm, key norm + page write
+        C = 2 * H * d + 2 * G * d + G * dv
+        zz = torch.randn(T, C + D, device=dev)
+        qn = torch.ones(d, device=dev)
+        qo = torch.empty(T, 2 * H * d, device=dev)
+        rot = _rot(att)
+
+        def qkv_path():
+            ops.head_norm_rope(zz, 2 * H, d, 0, d, qo, 0, d, meta, w=qn, eps=1e-6, rot=rot)
+            ops.head_norm_rope(zz, 2 * G, d, 2 * H * d, d, kc.view(-1, kc.shape[-1]), 0, d, meta, w=qn, eps=1e-6, rot=rot, row_map=meta["kv_slot"])
+            ops.head_norm_rope(zz, G, dv, 2 * (H + G) * d, dv, vc.view(-1, vc.shape[-1]), 0, dv, meta, row_map=meta["kv_slot"])
+        rec(f"{tag}/q k norm + rotation, k v page write", _timed(qkv_path, reps), 0, T * (C * 4 + 2 * H * d * 4 + (2 * G * d + G * dv) * es))
+        Ck = (H + 2 * G) * dk
+        zk = torch.randn(T, Ck, device=dev)
+        knw, qnw = torch.ones(G * dk, device=dev), torch.ones(H * dk, device=dev)
+
+        def kagolix_qkv():
+            ops.group_rmsnorm(zk[:, :H * dk], qnw, 1, 1e-6, out_dtype=dtype)
+            ops.kv_store(zk[:, H * dk:(H + G) * dk], knw, 1e-6, zk[:, (H + G) * dk:Ck], kk, kk, meta["kv_slot"])
+        rec(f"kagolix {tag}/query norm, key norm + page write", _timed(kagolix_qkv, reps), 0, T * (Ck * 4 + (H + 2 * G) * dk * es))
+        # the residual streams
+        xs, y = torch.randn(T, S * D, device=dev), torch.randn(T, D, device=dev)
+        hc = torch.cat([torch.full((S,), 1.0 / S), torch.ones(S), torch.eye(S).reshape(-1)]).to(dev)
+        nw = torch.ones(D, device=dev)
+        gate = zz[:, C:C + D]
+        rec(f"{tag}/streams sum + norm", _timed(lambda: ops.streams_norm(xs, hc, nw, 1e-6, dtype, S), reps), 0, T * D * (4 * S + es))
+        rec(f"{tag}/streams update, gated", _timed(lambda: ops.streams_update_(xs, y, gate, hc, 0.5, S), reps), 0, T * D * 4 * (2 * S + 2))
+        rec(f"{tag}/streams update, gated + next norm", _timed(lambda: ops.streams_update_norm_(xs, y, gate, hc, 0.5, S, hc, nw, 1e-6, dtype), reps),
+            0, T * D * (4 * (2 * S + 2) + es))
+        x = torch.randn(T, D, device=dev)
+        rec(f"kagolix {tag}/group norm", _timed(lambda: ops.group_rmsnorm(x, nw, 2, 1e-6, dtype), reps), 0, T * D * (4 + es))
+
+        def kagolix_add_norm():
+            ops.add_group_rmsnorm_(x, y, nw, 2, 1e-6)
+            ops.group_rmsnorm(x, nw, 2, 1e-6, dtype)
+        rec(f"kagolix {tag}/post-norm + residual add, group norm", _timed(kagolix_add_norm, reps), 0, T * D * (16 + es))
+        # the gated recurrence | Kagolix: the state-space scan
+        Hr, dr, dvr = rc["heads"], rc["dim"], rc["vdim"]
+        zr_ = torch.randn(T, 2 * Hr * dr + Hr * dvr, device=dev)
+        lower, mn = 0.9 * torch.rand(Hr * dr, device=dev), torch.ones(dvr, device=dev)
+        st = torch.zeros(B, Hr, dr, dvr, device=dev)
+        rec(f"{tag}/hgrn2 scan + head norm", _timed(lambda: ops.hgrn2_scan(zr_[:, :Hr * dr], zr_[:, Hr * dr:2 * Hr * dr], zr_[:, 2 * Hr * dr:], None,
+                                                                          lower, mn, st, meta, Hr, dr, dvr, 1e-6, dtype), reps),
+            6.0 * T * Hr * dr * dvr, T * (zr_.shape[1] * 4 + Hr * dvr * (8 + es)) + 2 * B * Hr * dr * dvr * 4)
+        nh, P, N = z["mh"], z["mp"], z["state"]
+        xbc = torch.randn(T, nh * P + 2 * N, device=dev)
+        z2, dt = torch.randn(T, nh * P, device=dev), torch.randn(T, nh, device=dev)
+        hp = torch.rand(nh, device=dev)
+        sst = torch.zeros(B, nh, N, P, device=dev)
+        rec(f"kagolix {tag}/ssd_scan", _timed(lambda: ops.ssd_scan(xbc, z2, dt, hp, hp * 0.3, hp, sst, meta, nh, P, N, 1), reps),
+            6.0 * T * nh * N * P, T * (xbc.shape[1] + 2 * nh * P + nh) * 4 + 2 * B * nh * N * P * 4)
+        # latent attention: the folded form over latent rows, and keys and values made per head for whole prompts
+        Hl, dn, drl, dvl, r = lat["heads"], lat["dim"], lat["rot_dim"], lat["vdim"], lat["kv_rank"]
+        pool = torch.randn(meta["n_pages"], ps, r + drl, device=dev).to(dtype)
+        qa = torch.randn(T, Hl * (r + drl), device=dev)
+        if tag == "decode":
+            rec(f"{tag}/latent attention (folded)", _timed(lambda: ops.attn_paged(
+                qa, pool, pool, meta, Hl, 1, r + drl, r, lat["scale"], 0.0, None, None, 0, ps, dtype), reps),
+                2.0 * T * keys * Hl * (2 * r + drl), B * keys * (r + drl) * es)
+        else:
+            kf = torch.randn(T, 1, Hl * (dn + drl), device=dev).to(dtype)
+            vf = torch.randn(T, 1, Hl * dvl, device=dev).to(dtype)
+            ql = torch.randn(T, Hl * (dn + drl), device=dev)
+            al = torch.empty(T, Hl * dvl, device=dev)
+            lm = dict(meta, page_table=meta["local_table"])
+            rec(f"{tag}/latent attention (keys and values unfolded)", _timed(lambda: ops.attn_paged(
+                ql, kf, vf, lm, Hl, Hl, dn + drl, dvl, lat["scale"], 0.0, None, None, 0, 1, dtype, out=al), reps),
+                2.0 * T * keys * Hl * (dn + drl + dvl))
+            g = torch.randn(T, Hl * dvl, device=dev)
+            rec(f"{tag}/sigmoid output gate", _timed(lambda: ops.sigmoid_gate(al, g, dtype), reps), 0, T * Hl * dvl * (8 + es))
+        # routing and the experts' activation
+        zr = torch.randn(T, E + D, device=dev)
+        logits = zr[:, :E]
+        gr = mlp["router"]["groups"]
+        rec(f"{tag}/grouped sigmoid routing", _timed(lambda: ops.moe_route_grouped(logits, top, gr["count"], gr["keep"], 2.0), reps), 0,
+            T * (E * 4 + top * 20))
+        corr = torch.zeros(E, device=dev)
+        rec(f"kagolix {tag}/corrected routing", _timed(lambda: ops.moe_route_corrected(logits, corr, top), reps), 0,
+            T * (E * 4 + top * 20))
+        up = torch.randn(T * top, ff, device=dev)
+        rec(f"{tag}/gelu (erf)", _timed(lambda: ops.unary(up, "gelu", dtype), reps), 0, T * top * ff * (4 + es))
+        gu = torch.randn(T * top, 2 * ff, device=dev)
+        rec(f"kagolix {tag}/silu gate product", _timed(lambda: ops.gate_mul(gu, dtype, "silu"), reps), 0, T * top * ff * (8 + es))
+        route = ops.moe_route_grouped(logits, top, gr["count"], gr["keep"], 2.0)
+        yo = torch.randn(T * top, D, device=dev)
+        rec(f"{tag}/expert sum", _timed(lambda: ops.moe_weighted_sum(yo, route), reps), 0, T * D * 4 * (top + 1))
+        h = torch.randn(T, D, device=dev).to(dtype)
+        n_in = C + D
+        w = (0.02 * torch.randn(n_in, D, device=dev)).to(dtype)
+        rec(f"{tag}/gemm {T}x{n_in}x{D}", _timed(lambda: ops.matmul_nt(h, w), reps), 2.0 * T * n_in * D,
+            es * (n_in * D + T * D) + 4 * T * n_in)
+    return {"part": "kernels", "family": "lopilix", "dtype": str(dtype), "batch": B, "context": L, "kernels": res}
+
+
 def main(a) -> int:
     """``bench.py --hybrid SIZE`` (one GPU)."""
     dev = torch.device("cuda", 0)
@@ -551,6 +723,20 @@ def main(a) -> int:
     B, L = a.hybrid_batch, a.hybrid_context
     lines: List[dict] = []
     parts = a.hybrid_parts.split(",")
+    if getattr(a, "hybrid_family", "kagolix") == "lopilix":
+        if "hybrid" in parts:
+            lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev, lopilix_config(z), "lopilix"))
+            print(json.dumps(lines[-1]), flush=True)
+        if "dense" in parts:      # (the closest existing model: the Kagolix stack of attention, recurrent and state-space layers)
+            lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev, hybrid_config(z), "kagolix"))
+            print(json.dumps(lines[-1]), flush=True)
+        if "kernels" in parts:
+            lines.append(bench_lopilix_kernels(z, dtype, B, L, dev))
+            print(json.dumps(lines[-1]), flush=True)
+        if a.json_out:
+            with open(a.json_out, "w") as f:
+                json.dump(lines, f, indent=1)
+        return 0
     if getattr(a, "hybrid_family", "kagolix") == "gizezen":
         if "hybrid" in parts:
             lines.append(bench_hybrid_model(z, dtype, B, L, a.steps * 8, dev, gizezen_config(z), "gizezen"))

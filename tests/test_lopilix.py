@@ -521,3 +521,21 @@ def test_trace_run_program_replays_steps(tmp_path):
     got = np.concatenate([np.fromfile(out / "0.f32", dtype="<f4").reshape(3, -1), np.fromfile(out / "2.f32", dtype="<f4").reshape(2, -1)])
     assert not (out / "1.f32").exists()
     assert lu.rel_err(got, np.concatenate([wa[[0, 6]], wb[[0]], wa[[8]], wb[[2]]])) < TOL
+
+
+def test_bench_model_builder_runs_on_cpu():
+    """The benchmark's synthetic stack (bench.py --hybrid --hybrid-family lopilix) at a toy size: random layer
+    images straight into a host store, a prompt step and a decode step through the runner."""
+    from flexible_llm_sharding_amd.engine import ShardedRunner
+    from flexible_llm_sharding_amd.utils.hybrid_bench import lopilix_config, synthetic_hybrid_store
+    z = dict(width=64, heads=4, kv=2, dim=16, ff=96, experts=4, top=2, eff=16, blocks=2, mh=2, mp=8, state=8, chunk=12, vocab=50)
+    cfg = lopilix_config(z, times=2, streams=2)
+    assert len(cfg.layer_names()) == 9
+    src = synthetic_hybrid_store(cfg, "cpu", torch.float32)
+    r = ShardedRunner(cfg, src, device="cpu", layer_num_per_shard=2, storage_location="cpu", compute_dtype=torch.float32,
+                      state_tokens=64, state_seqs=2)
+    out = r.step([StepEntry("a", list(range(20)), [19]), StepEntry("b", [1, 2, 3], [2])])
+    assert out[0][0].shape == (1, 50) and np.isfinite(out[0][0]).all() and np.isfinite(out[1][0]).all()
+    out = r.step([StepEntry("a", [5], [0]), StepEntry("b", [6], [])], ["a", "b"])
+    assert out[1] is None and np.isfinite(out[0][0]).all() and not r.seq_cache.requests
+    r.close()
