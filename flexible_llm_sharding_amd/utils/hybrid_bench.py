@@ -209,7 +209,7 @@ def bench_hybrid_model(z: dict, dtype, B: int, L: int, steps: int, dev, cfg=None
         r.step([StepEntry(i, [7], [0]) for i in ids])
     decode()
     t_dec = _timed(decode, steps)
-    out = {"part": part, "model": f"{cfg.family} {cfg.total_params() / 1e9:.2f}B params, {len(cfg.layers)} layers, width {cfg.width}",
+    out = {"part": part, "model": f"{cfg.family} {cfg.total_params() / 1e9:.2f}B params, {cfg.num_hidden_layers} layer runs, width {cfg.width}",
            "dtype": str(dtype), "batch": B, "context": L, "prefill_tok_s": B * L / t_pre, "prefill_ms": t_pre * 1e3,
            "decode_tok_s": B / t_dec, "decode_ms_per_step": t_dec * 1e3, "state_bytes": r.seq_cache.nbytes()}
     r.close()
@@ -628,9 +628,7 @@ def bench_lopilix_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
         rot = _rot(att)
 
         def qkv_path():
-            ops.head_norm_rope(zz, 2 * H, d, 0, d, qo, 0, d, meta, w=qn, eps=1e-6, rot=rot)
-            ops.head_norm_rope(zz, 2 * G, d, 2 * H * d, d, kc.view(-1, kc.shape[-1]), 0, d, meta, w=qn, eps=1e-6, rot=rot, row_map=meta["kv_slot"])
-            ops.head_norm_rope(zz, G, dv, 2 * (H + G) * d, dv, vc.view(-1, vc.shape[-1]), 0, dv, meta, row_map=meta["kv_slot"])
+            ops.qkv_conv_rope_store(zz, None, None, meta, 2 * H, 2 * G, d, dv, qo, kc, vc, eps=1e-6, rot=rot, v_heads=G, q_norm=qn, k_norm=qn)
         rec(f"{tag}/q k norm + rotation, k v page write", _timed(qkv_path, reps), 0, T * (C * 4 + 2 * H * d * 4 + (2 * G * d + G * dv) * es))
         Ck = (H + 2 * G) * dk
         zk = torch.randn(T, Ck, device=dev)

@@ -36,7 +36,7 @@ def main():
     a = ap.parse_args()
     c = sqlite3.connect(a.db)
     rows = c.execute("select name, start, end from kernels order by start").fetchall()
-    starts = [i for i, r in enumerate(rows) if "embed_kernel" in r[0]][::a.embeds_per_pass]
+    starts = [i for i, r in enumerate(rows) if "embed_kernel" in r[0] or "embed_pos_kernel" in r[0]][::a.embeds_per_pass]
     passes = []
     for j, i0 in enumerate(starts):
         i1 = starts[j + 1] if j + 1 < len(starts) else len(rows)

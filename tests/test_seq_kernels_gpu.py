@@ -670,3 +670,29 @@ def test_grouped_sigmoid_routing(ops, T, E, top, groups, keep):
     offs, dest = a.offs.cpu().long(), a.dest.cpu().long()
     assert bool(((dest >= offs[a.ids.cpu().long()]) & (dest < offs[a.ids.cpu().long() + 1])).all())
     assert torch.equal(a.rows.cpu().long()[dest], torch.arange(T)[:, None].expand(T, top))
+
+
+@pytest.mark.parametrize("cdt,tol", DTYPES)
+@pytest.mark.parametrize("Hh,G,Gv,d,dv,rot", [(12, 4, 2, 10, 14, (6, 50.0)), (8, 4, 2, 64, 128, (32, 1e6)), (2, 2, 1, 32, 64, (32, 1e4)),
+                                              (4, 2, 1, 130, 70, None)])
+def test_projected_rows_with_weighted_norms_before_the_rotation(ops, cdt, tol, Hh, G, Gv, d, dv, rot):
+    """The one-pass kernel in its second form: q and k heads RMS-normed with a weight before the rotation, fewer
+    value heads than key heads in the row, no convolution; against the chain of plain ops."""
+    H, R = ops
+    torch.manual_seed(21)
+    C = Hh * d + G * d + Gv * dv
+    qw, kw_ = 1 + 0.3 * torch.randn(d, device=DEV), 1 + 0.3 * torch.randn(d, device=DEV)
+    for lens, pos0 in (([1, 40, 3, 130], [900, 0, 17, 2000]), ([1, 1, 1], [5, 0, 300])):
+        md, n_pages, _ = meta_of(lens, pos0, DEV)
+        T = sum(lens)
+        z = torch.randn(T, C + 7, device=DEV)
+        outs = []
+        for O in (H, R):
+            q = torch.zeros(T, Hh * d, device=DEV)
+            kc = torch.zeros(n_pages, 16, G * d, device=DEV, dtype=cdt)
+            vc = torch.zeros(n_pages, 16, Gv * dv, device=DEV, dtype=cdt)
+            O.qkv_conv_rope_store(z, None, None, md, Hh, G, d, dv, q, kc, vc, eps=1e-5, rot=rot, v_heads=Gv, q_norm=qw, k_norm=kw_)
+            outs.append((q, kc, vc))
+        close(outs[0][0], outs[1][0], 3e-4)
+        close(outs[0][1], outs[1][1], max(tol, 3e-4))
+        close(outs[0][2], outs[1][2], tol)
