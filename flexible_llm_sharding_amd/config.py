@@ -827,6 +827,9 @@ class LopilixConfig:
                     raise NotImplementedError(f"layer {i}: latent rows above 512 + 512")
             if max(int(m["dim"]), int(m["vdim"])) > 512:
                 raise NotImplementedError(f"layer {i}: head sizes above 512")
+            if l.type == "hgrn2" and int(m["dim"]) > 256:
+                # (the scan keeps a value column's state rows in the registers of 16 lanes, 16 rows each)
+                raise NotImplementedError(f"layer {i}: a recurrent state of more than 256 rows per head")
             if l.mlp is not None:
                 if l.mlp["kind"] not in ("dense", "moe"):
                     raise NotImplementedError(f"layer {i}: mlp kind {l.mlp['kind']!r}")
@@ -835,6 +838,8 @@ class LopilixConfig:
                     if not 1 <= r["top"] <= min(r["experts"], 16) or r["experts"] > 1024:
                         raise NotImplementedError(f"layer {i}: router {r}")
                     g = r.get("groups")
+                    if g and int(g["count"]) > 64:
+                        raise NotImplementedError(f"layer {i}: more than 64 expert groups")
                     if g and (r["experts"] % int(g["count"]) or not 1 <= int(g["keep"]) <= int(g["count"])
                               or int(g["keep"]) * (r["experts"] // int(g["count"])) < r["top"]):
                         raise ValueError(f"layer {i}: router groups {g} do not fit {r['experts']} experts, top {r['top']}")
