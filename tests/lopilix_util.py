@@ -118,13 +118,18 @@ def oracle_logits(cfg, sd, tokens, trace=None):
     return oracle.forward(f64(sd), cfg, list(tokens), trace).numpy()
 
 
-def rel_err(got, want):
-    """Mean-free RMS difference of logit rows over the RMS of the wanted rows (the worst row)."""
+def row_errs(got, want):
+    """Per row: mean-free RMS difference of the logits over the RMS of the wanted row."""
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     d = got - want
     d = d - d.mean(-1, keepdims=True)
     w = want - want.mean(-1, keepdims=True)
-    return float((np.sqrt((d ** 2).mean(-1)) / (np.sqrt((w ** 2).mean(-1)) + 1e-12)).max())
+    return np.sqrt((d ** 2).mean(-1)) / (np.sqrt((w ** 2).mean(-1)) + 1e-12)
+
+
+def rel_err(got, want):
+    """The worst row of ``row_errs``."""
+    return float(row_errs(got, want).max())
 
 
 def tokens(n, vocab, seed):

@@ -302,9 +302,11 @@ def test_head_sizes_of_the_matrix_core_kernels(tmp_path, device):
     want = lu.oracle_logits(cfg, sd, toks)
     whole = run_cut(runner, "a", toks, [230])
     cut = run_cut(runner, "b", toks, [150, 40])
-    # (the difference of two attention maps, divided by its own root mean square, amplifies the rounding of both)
-    assert lu.rel_err(whole, want) < 0.16 and lu.rel_err(cut, want) < 0.16
-    assert lu.rel_err(cut, whole) < 0.12
+    # (the difference of two attention maps, divided by its own root mean square, amplifies the rounding of both where
+    # the maps nearly cancel: a few rows stand far above the rest, so the bound is on the mean and on nine rows in ten)
+    for got, ref, mean, q90 in ((whole, want, 0.05, 0.08), (cut, want, 0.05, 0.08), (cut, whole, 0.05, 0.08)):
+        e = lu.row_errs(got, ref)
+        assert e.mean() < mean and np.quantile(e, 0.9) < q90, (e.mean(), np.quantile(e, 0.9))
     runner.close()
 
 
