@@ -361,6 +361,36 @@ def main(argv=None):
     mine = sorted({i for sh in plan.my_shards for i in sh})
     t0 = time.perf_counter()
     prog = lambda i, n: log(rank, f"[bench]   layer {i}/{n} ({time.perf_counter() - t0:.0f}s)") if i % 10 == 0 else None  # noqa: E731
+    store = None
+    if a.weights == "host":
+        # the whole model pinned in host RAM; a box whose driver pins less than the model holds (hipHostMalloc fails
+        # although RAM is free) gets the layer-file streamer instead, which pins a 256 MB ring
+        short = 0.0
+        try:
+            log(rank, f"[bench] generating {len(mine)} random-init {a.model} layers on {dev} -> pinned host ...")
+            if dp:
+                # scatter-load: this rank keeps 1/G of every layer; layers re-assembled by RCCL all-gather
+                store = SlicedHostStore.synthetic(cfg, dev, rank, world, seed=a.seed, names=[names[i] for i in mine],
+                                                  progress=prog, fold_norms=fold)
+            else:
+                store = HostStore.synthetic(cfg, dev, seed=a.seed, names=[names[i] for i in mine], progress=prog,
+                                            fold_norms=fold)
+            log(rank, f"[bench] host store {store.total_bytes / 1e9:.1f} GB in {time.perf_counter() - t0:.1f}s")
+            data_w = f"random-init {a.model} weights in {'HBM (resident)' if a.resident else 'pinned host RAM'}"
+
+        except (RuntimeError, MemoryError) as e:
+            if "out of memory" not in str(e).lower():
+                raise
+            short = 1.0
+            log(rank, f"[bench] pinned host memory ran out ({type(e).__name__}); streaming per-layer files instead")
+        if comm.all_reduce_max(short) > 0:
+            store = None
+            import gc
+            gc.collect()
+            if not a.cpu:
+                torch.cuda.empty_cache()
+            a.weights = "stream"
+            fold = False                 # (the layer-file path folds the norm weights as each layer lands)
     if a.weights == "stream":
         ckpt = a.ckpt_dir or f"/tmp/fls_bench_ckpt_{a.model}{'' if a.num_layers is None else f'-L{a.num_layers}'}_{a.ckpt_dtype}_u{a.unique_layers}"
         log(rank, f"[bench] per-layer checkpoint {ckpt} (unique decoder layers: {a.unique_layers}) ...")
@@ -376,18 +406,6 @@ def main(argv=None):
         data_w = (f"random-init {a.model} weights as per-layer {a.ckpt_dtype} safetensors files "
                   f"({a.unique_layers} distinct decoder layers, the rest hard links), streamed from the files "
                   f"every pass ({'O_DIRECT' if a.o_direct else 'page cache'})")
-    else:
-        log(rank, f"[bench] generating {len(mine)} random-init {a.model} layers on {dev} -> pinned host ...")
-        if dp:
-            # scatter-load: this rank keeps 1/G of every layer; layers re-assembled by RCCL all-gather
-            store = SlicedHostStore.synthetic(cfg, dev, rank, world, seed=a.seed, names=[names[i] for i in mine],
-                                              progress=prog, fold_norms=fold)
-        else:
-            store = HostStore.synthetic(cfg, dev, seed=a.seed, names=[names[i] for i in mine], progress=prog,
-                                        fold_norms=fold)
-        log(rank, f"[bench] host store {store.total_bytes / 1e9:.1f} GB in {time.perf_counter() - t0:.1f}s")
-        data_w = f"random-init {a.model} weights in {'HBM (resident)' if a.resident else 'pinned host RAM'}"
-
     if not a.cpu:
         torch.cuda.empty_cache()     # set-up only: the weight generator's staging blocks are not part of a pass
     tok_dir = f"/tmp/fls_bench_tok_{os.getpid()}"
