@@ -198,9 +198,15 @@ def _diff_attention(ctx, L, W, h, meta, name: str):
     kc, vc = ctx.cache.kv(name)
     rot = _rot(m)
     q = torch.empty(T, 2 * H * d, dtype=torch.float32, device=z.device)
-    # per head and map: norm with the shared weight, rotation; q to fp32 rows, k and v into their pages, one pass
-    ops.qkv_conv_rope_store(z, None, None, meta, 2 * H, 2 * G, d, dv, q, kc, vc, eps=eps, rot=rot, v_heads=G, q_norm=W["qn"],
-                            k_norm=W["kn"])
+    # per head and map: norm with the shared weight, rotation; q to fp32 rows, k and v into their pages
+    if rot is None or rot[2] is None:
+        ops.qkv_conv_rope_store(z, None, None, meta, 2 * H, 2 * G, d, dv, q, kc, vc, eps=eps, rot=rot, v_heads=G, q_norm=W["qn"],
+                                k_norm=W["kn"])                              # (one pass)
+    else:       # rescaled frequencies carry an amplitude on cosines and sines, which the per-head op applies
+        ops.head_norm_rope(z, 2 * H, d, 0, d, q, 0, d, meta, w=W["qn"], eps=eps, rot=rot)
+        ops.head_norm_rope(z, 2 * G, d, c["k"][0], d, kc.view(-1, kc.shape[-1]), 0, d, meta, w=W["kn"], eps=eps, rot=rot,
+                           row_map=meta["kv_slot"])
+        ops.head_norm_rope(z, G, dv, c["v"][0], dv, vc.view(-1, vc.shape[-1]), 0, dv, meta, row_map=meta["kv_slot"])
     # the two maps as 2 H heads over 2 G key heads; both maps of a key head read the same value head
     a = torch.empty(T, 2 * H * dv, dtype=torch.float32, device=z.device)
     ops.attn_paged(q, kc, vc, meta, 2 * H, 2 * G, d, dv, scale=float(m["scale"]), softcap=0.0, r1=None, r2=None, chunk=0,

@@ -14,10 +14,12 @@ from flexible_llm_sharding_amd.utils.safetensors_io import save_file
 SCALING = {"factor": 3.0, "original": 24, "fast": 4.0, "slow": 0.5}
 
 
-def attn(heads=6, kv_heads=2, dim=10, vdim=14, rot_dims=6, base=50.0, scale=0.4, diff=0.25):
+def attn(heads=6, kv_heads=2, dim=10, vdim=14, rot_dims=6, base=50.0, scale=0.4, diff=0.25, scaling=None):
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "diff": diff}
     if rot_dims:
         m["rot"] = {"dims": rot_dims, "base": base}
+        if scaling is not None:
+            m["rot"]["scaling"] = dict(scaling)
     return ("attention", m)
 
 

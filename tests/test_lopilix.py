@@ -74,6 +74,7 @@ LOOP = (1, 4, 2)
     ("differential-attention", [(lu.attn(scale=1.5), None)], {}),
     ("differential-attention-one-head-no-rotation", [(lu.attn(heads=1, kv_heads=1, dim=4, vdim=3, rot_dims=0), None)], {}),
     ("differential-attention-multi-head-full-rotation", [(lu.attn(heads=3, kv_heads=3, dim=8, vdim=8, rot_dims=8), None)], {}),
+    ("differential-attention-rescaled-rotation", [(lu.attn(scaling=lu.SCALING), None)], {}),
     ("hgrn2", [(lu.hgrn(), None)], {}),
     ("hgrn2-one-head-wide-state", [(lu.hgrn(heads=1, dim=37, vdim=70), None)], {}),
     ("hgrn2-narrow", [(lu.hgrn(heads=5, dim=1, vdim=1), None)], {}),
