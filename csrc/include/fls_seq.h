@@ -167,11 +167,10 @@ int fls_seq_streams_norm(const float* xs, int ldx, const int* idx, const float* 
                          int rows, int D, int S, float eps, fls_stream_t s);
 // all streams at once from the old ones: xs[t, r] <- sum_s mix[s, r] xs[t, s] + mult * out[r] * y[t] * sigmoid(gate[t]);
 // hc = [in (S) | out (S) | mix (S x S, [from, to])] (nullable: S = 1, out = mix = 1); gate nullable.  h != null: also
-// h[t] = the norm above of the NEW streams with coefficients ncoef (nullable) and weight nw, type th.  dest != null
-// ([rows, top] with weights rw, top <= 16): y holds a mixture's expert rows and y[t] stands for sum_k rw[t, k] y[dest[t, k]]
+// h[t] = the norm above of the NEW streams with coefficients ncoef (nullable) and weight nw, type th
 int fls_seq_streams_update(float* xs, int ldx, const float* y, int ldy, const float* gate, int ldg, const float* hc, float mult,
                            int rows, int D, int S, const float* ncoef, const float* nw, void* h, int th, int ldh, float eps,
-                           const int* dest, const float* rw, int top, fls_stream_t s);
+                           fls_stream_t s);
 int fls_seq_scale(float* z, int ldz, int rows, int cols, float alpha, fls_stream_t s);
 // y = o * sigmoid(g); o of type to_, y of type ty
 int fls_seq_sigmoid_gate(const void* o, int to_, int ldo, const float* g, int ldg, void* y, int ty, int ldy, int rows, int cols,

@@ -664,4 +664,4 @@ extern "C" int fls_seq_moe_combine(float* x, int ldx, const float* y, int ldy, c
   return 0;
 }
 
-extern "C" int fls_seq_version(void) { return 11; }
+extern "C" int fls_seq_version(void) { return 10; }

@@ -5,7 +5,6 @@
 #include "fls_seq.h"
 
 #define MAX_STREAMS 8
-#define SU_MAX_TOP 16          // choices per token of a mixture whose sum joins the streams
 
 // ------------------------------------------------------------------------------- embedding
 // out[t, c * D + j] = table[ids[t], j] * scale + pos_table[tok_pos[t], j] for every copy c
@@ -109,23 +108,15 @@ extern "C" int fls_seq_streams_norm(const float* xs, int ldx, const int* idx, co
 // ------------------------------------------------------------------------ streams update (+ next norm)
 // one block per row.  Per column: the S old values, the gated sublayer output g = y sigmoid(gate), the S new
 // values mix^T old + mult out g, written back; with NORM also u = sum_s ncoef[s] new_s, whose norm is the next
-// sublayer's input.  Columns <= 256 * SN_PIECES keep u in registers between the two halves.  dest != null: y holds the
-// rows of a mixture's experts and the sublayer output is their weighted sum, y_t = sum_k rw[t, k] y[dest[t, k]].
+// sublayer's input.  Columns <= 256 * SN_PIECES keep u in registers between the two halves.
 template <typename TO, int NORM>
 __global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__ xs, int ldx, const float* __restrict__ y, int ldy,
                                                              const float* __restrict__ gate, int ldg,
                                                              const float* __restrict__ hc, float mult, int D, int S,
                                                              const float* __restrict__ ncoef, const float* __restrict__ nw,
-                                                             TO* __restrict__ h, int ldh, float eps,
-                                                             const int* __restrict__ dest, const float* __restrict__ rw, int top) {
+                                                             TO* __restrict__ h, int ldh, float eps) {
   __shared__ float red[4];
   __shared__ float mixs[MAX_STREAMS * MAX_STREAMS], outs[MAX_STREAMS], ncs[MAX_STREAMS];
-  __shared__ float rws[SU_MAX_TOP];
-  __shared__ int dests[SU_MAX_TOP];
-  if (dest != nullptr && (int)threadIdx.x < top) {
-    dests[threadIdx.x] = dest[(size_t)blockIdx.x * top + threadIdx.x];
-    rws[threadIdx.x] = rw[(size_t)blockIdx.x * top + threadIdx.x];
-  }
   if (threadIdx.x < S * S) mixs[threadIdx.x] = hc != nullptr ? hc[2 * S + threadIdx.x] : 1.f;
   if (threadIdx.x < S) {
     outs[threadIdx.x] = mult * (hc != nullptr ? hc[S + threadIdx.x] : 1.f);
@@ -144,13 +135,7 @@ __global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__
     float old[MAX_STREAMS];
 #pragma unroll
     for (int s = 0; s < MAX_STREAMS; ++s) old[s] = s < S ? xr[(size_t)s * D + c] : 0.f;
-    float g;
-    if (dest != nullptr) {
-      g = 0.f;
-      for (int k = 0; k < top; ++k) g += rws[k] * y[(size_t)dests[k] * ldy + c];
-    } else {
-      g = yr[c];
-    }
+    float g = yr[c];
     if (gr != nullptr) g *= sigmoid_f(gr[c]);
     float un = 0.f;
 #pragma unroll
@@ -196,13 +181,12 @@ __global__ __launch_bounds__(256) void streams_update_kernel(float* __restrict__
 
 extern "C" int fls_seq_streams_update(float* xs, int ldx, const float* y, int ldy, const float* gate, int ldg, const float* hc,
                                       float mult, int rows, int D, int S, const float* ncoef, const float* nw, void* h, int th,
-                                      int ldh, float eps, const int* dest, const float* rw, int top, fls_stream_t s) {
+                                      int ldh, float eps, fls_stream_t s) {
   if (rows <= 0) return 0;
-  if (dest != nullptr && (rw == nullptr || top < 1 || top > SU_MAX_TOP)) return -1;
   if (S < 1 || S > MAX_STREAMS || ldx < S * D || (hc == nullptr && S != 1) || (h != nullptr && nw == nullptr)) return -1;
   hipStream_t st = (hipStream_t)s;
 #define SU(TO, N) hipLaunchKernelGGL((streams_update_kernel<TO, N>), dim3(rows), dim3(256), 0, st, xs, ldx, y, ldy, gate, ldg, hc, mult, \
-                                     D, S, ncoef, nw, (TO*)h, ldh, eps, dest, rw, top)
+                                     D, S, ncoef, nw, (TO*)h, ldh, eps)
   if (h == nullptr) SU(float, 0);
   else if (th == 1) SU(bf16_t, 1);
   else SU(float, 1);

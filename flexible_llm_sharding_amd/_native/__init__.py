@@ -130,7 +130,7 @@ def _load_kernels(path: str = _KERNELS):
     return lib
 
 
-SEQ_ABI = 11   # csrc/include/fls_seq.h
+SEQ_ABI = 10   # csrc/include/fls_seq.h
 
 
 def _load_seq():
@@ -173,7 +173,7 @@ def _load_seq():
     _bind(lib, "fls_seq_moe_route_grouped", i, p, i, i, i, i, i, i, f, p, p, p, p)
     _bind(lib, "fls_seq_embed_pos", i, p, p, i, p, p, p, i, i, i, i, f, i, p)
     _bind(lib, "fls_seq_streams_norm", i, p, i, p, p, p, p, i, i, i, i, i, f, p)
-    _bind(lib, "fls_seq_streams_update", i, p, i, p, i, p, i, p, f, i, i, i, p, p, p, i, i, f, p, p, i, p)
+    _bind(lib, "fls_seq_streams_update", i, p, i, p, i, p, i, p, f, i, i, i, p, p, p, i, i, f, p)
     _bind(lib, "fls_seq_scale", i, p, i, i, i, f, p)
     _bind(lib, "fls_seq_sigmoid_gate", i, p, i, i, p, i, p, i, i, i, i, p)
     _bind(lib, "fls_seq_diff_combine", i, p, i, p, i, f, i, i, f, p, i, i, i, p)

@@ -272,7 +272,7 @@ def _dense(ctx, mlp: dict, W, h):
     ff = int(mlp["ff"])
     z = ops.matmul_nt(h, W["wgu"], bias=W["bgu"])                          # fp32 [T, gate | up | residual gate]
     y = ops.matmul_nt(ops.gate_mul(z[:, :2 * ff], cdt, act="silu"), W["wdown"], bias=W["bdown"])
-    return y, _gate_cols(ctx.cfg, z, 2 * ff), None
+    return y, _gate_cols(ctx.cfg, z, 2 * ff)
 
 
 def _moe(ctx, mlp: dict, W, h):
@@ -285,7 +285,7 @@ def _moe(ctx, mlp: dict, W, h):
     hp = ops.gather_rows(h, route.rows)                                   # rows sorted by expert
     up = ops.grouped_matmul_nt(hp, W["wup"], route.offs)                  # fp32 [T top, ff]
     yo = ops.grouped_matmul_nt(ops.unary(up, "gelu", cdt), W["wdown"], route.offs)
-    return yo, _gate_cols(ctx.cfg, z, E), route                          # (the experts' rows: the streams' update sums them)
+    return ops.moe_weighted_sum(yo, route), _gate_cols(ctx.cfg, z, E)
 
 
 _MIXERS = {"attention": _diff_attention, "hgrn2": _hgrn2, "latent_attention": _latent_attention}
@@ -302,8 +302,8 @@ def run_block(ctx, W, xs: torch.Tensor, meta: dict, name: str) -> torch.Tensor:
         return ops.streams_update_(xs, y, gate, hc1, mult, S)
     # (the streams' update and the feed-forward's norm read and write the streams once)
     h = ops.streams_update_norm_(xs, y, gate, hc1, mult, S, hc2, W["norm2"], eps, cdt)
-    y, gate, route = (_dense if L.mlp["kind"] == "dense" else _moe)(ctx, L.mlp, W, h)
-    return ops.streams_update_(xs, y, gate, hc2, mult, S, route=route)
+    y, gate = (_dense if L.mlp["kind"] == "dense" else _moe)(ctx, L.mlp, W, h)
+    return ops.streams_update_(xs, y, gate, hc2, mult, S)
 
 
 def run_layer(ctx, name: str, W: Dict[str, torch.Tensor], state, batch, meta: dict) -> torch.Tensor:

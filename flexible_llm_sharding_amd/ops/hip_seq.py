@@ -155,15 +155,10 @@ class HipSeqOps:
                                          _CODE[out_dtype], D, rows, D, streams, float(eps), _stream()), "fls_seq_streams_norm")
         return y
 
-    def _streams_update(self, xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype, route=None):
+    def _streams_update(self, xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype):
         _rows(xs, "xs", torch.float32)
         _rows(y, "y", torch.float32)
-        T, D = xs.shape[0], y.shape[1]
-        if route is not None:
-            if tuple(route.dest.shape) != (T, route.top) or y.shape[0] != T * route.top or route.top > 16:
-                raise ValueError("streams_update_: the experts' rows do not fit the routing")
-        elif y.shape[0] != T:
-            raise ValueError("streams_update_: y has other rows than xs")
+        T, D = y.shape
         if tuple(xs.shape) != (T, streams * D):
             raise ValueError("streams_update_: xs must be [T, streams * D]")
         if gate is not None:
@@ -185,19 +180,16 @@ class HipSeqOps:
                                            hc.data_ptr() if hc is not None else None, float(mult), T, D, streams,
                                            coef.data_ptr() if (w is not None and coef is not None) else None,
                                            w.data_ptr() if w is not None else None, h.data_ptr() if h is not None else None,
-                                           _CODE[out_dtype] if h is not None else 0, D, float(eps),
-                                           route.dest.data_ptr() if route is not None else None,
-                                           route.w.data_ptr() if route is not None else None,
-                                           route.top if route is not None else 0, _stream()),
+                                           _CODE[out_dtype] if h is not None else 0, D, float(eps), _stream()),
              "fls_seq_streams_update")
         return h
 
-    def streams_update_(self, xs, y, gate, hc, mult, streams, route=None):
-        self._streams_update(xs, y, gate, hc, mult, streams, None, None, 0.0, torch.float32, route)
+    def streams_update_(self, xs, y, gate, hc, mult, streams):
+        self._streams_update(xs, y, gate, hc, mult, streams, None, None, 0.0, torch.float32)
         return xs
 
-    def streams_update_norm_(self, xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype, route=None):
-        return self._streams_update(xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype, route)
+    def streams_update_norm_(self, xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype):
+        return self._streams_update(xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype)
 
     def scale_(self, z, alpha):
         _rows(z, "z", torch.float32)

@@ -83,13 +83,10 @@ class TorchSeqOps:
         u = x3.sum(1) if coef is None else torch.einsum("s,tsd->td", coef.float()[:streams], x3)
         return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
 
-    def streams_update_(self, xs, y, gate, hc, mult, streams, route=None):
+    def streams_update_(self, xs, y, gate, hc, mult, streams):
         """All streams at once from the old ones: xs_t <- sum_s mix[s, t] xs_s + mult * out[t] * y * sigmoid(gate).
         ``hc`` = [in (streams) | out (streams) | mix (streams x streams, [from, to])] fp32, None: one stream
-        that keeps itself (a plain residual sum); ``gate`` [T, D] fp32 logits or None.  ``route``: y holds the rows
-        of a mixture's experts ([T top, D], sorted by expert) and stands for their weighted sum per token."""
-        if route is not None:
-            y = self.moe_weighted_sum(y, route)
+        that keeps itself (a plain residual sum); ``gate`` [T, D] fp32 logits or None."""
         T = xs.shape[0]
         x3 = xs.reshape(T, streams, xs.shape[1] // streams)
         yy = y.float()
@@ -103,9 +100,9 @@ class TorchSeqOps:
         xs.copy_(new.reshape(T, -1))
         return xs
 
-    def streams_update_norm_(self, xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype, route=None):
+    def streams_update_norm_(self, xs, y, gate, hc, mult, streams, coef, w, eps, out_dtype):
         """``streams_update_`` and the next sublayer's ``streams_norm`` of the new streams, in one pass."""
-        self.streams_update_(xs, y, gate, hc, mult, streams, route)
+        self.streams_update_(xs, y, gate, hc, mult, streams)
         return self.streams_norm(xs, coef, w, eps, out_dtype, streams)
 
     def scale_(self, z, alpha):

@@ -703,12 +703,7 @@ def bench_lopilix_kernels(z: dict, dtype, B: int, L: int, dev) -> dict:
         rec(f"kagolix {tag}/silu gate product", _timed(lambda: ops.gate_mul(gu, dtype, "silu"), reps), 0, T * top * ff * (8 + es))
         route = ops.moe_route_grouped(logits, top, gr["count"], gr["keep"], 2.0)
         yo = torch.randn(T * top, D, device=dev)
-        rec(f"{tag}/expert sum + streams update, gated", _timed(lambda: ops.streams_update_(xs, yo, gate, hc, 0.5, S, route=route), reps), 0,
-            T * D * 4 * (2 * S + 1 + top))
-
-        def kagolix_combine():
-            ops.add_group_rmsnorm_(x, ops.moe_weighted_sum(yo, route), nw, 2, 1e-6)
-        rec(f"kagolix {tag}/expert sum, post-norm + residual add", _timed(kagolix_combine, reps), 0, T * D * 4 * (top + 5))
+        rec(f"{tag}/expert sum", _timed(lambda: ops.moe_weighted_sum(yo, route), reps), 0, T * D * 4 * (top + 1))
         h = torch.randn(T, D, device=dev).to(dtype)
         n_in = C + D
         w = (0.02 * torch.randn(n_in, D, device=dev)).to(dtype)
